@@ -1,0 +1,99 @@
+/* jf_layers.h — C ABI of libjf_layers.so: layer kernels for decoders with a 32-bit residual stream, served over a paged
+ * key/value pool and per-request state slots.  Device pointers + sizes, stream as void*.  Activation tensors are row-major
+ * float or bfloat16 (`dtype`: JL_F32 / JL_BF16) with an explicit row stride in elements where a tensor is a column range of a
+ * wider matrix; residual stream, router, probabilities and recurrent state are float.  Every function returns JL_OK or a
+ * negative code (jl_last_error() has the text) and only enqueues work on `stream`.
+ *
+ * A step's tokens are one ragged batch: N token rows, the rows of one request consecutive and in position order.  Per request
+ * b the int32 record seq[b] = {row0, count, pos0, slot}: its first row, its number of rows, the position of its first row
+ * (= tokens already cached) and its state slot. */
+#ifndef JF_LAYERS_H
+#define JF_LAYERS_H
+
+#include <stdint.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+#define JL_API __attribute__((visibility("default")))
+#define JL_VERSION 100
+#define JL_OK 0
+#define JL_E_INVALID (-1)
+#define JL_E_LAUNCH (-3)
+#define JL_F32 0
+#define JL_BF16 1
+
+JL_API int jl_version(void);
+JL_API const char *jl_last_error(void);
+
+/* x[n, :] = embed[ids[n], :] * scale (float); x0, when given, receives the same rows (the embedding output a repeated pass adds
+ * again). */
+JL_API int jl_embed_scale(const void *embed, int dtype, const int64_t *ids, int64_t N, int32_t W, float scale, float *x, float *x0,
+                          void *stream);
+
+/* Residual update + RMS norm: x[n] += sum_{s < y_count} y[n * y_count + s] (y of dtype y_dtype, may be null) + x0[n] (float,
+ * may be null); then, when `out` is given, out[n] = x[n] / sqrt(mean(x[n]^2) + eps) * w (w of `dtype`, null = no weight). */
+JL_API int jl_add_rmsnorm(float *x, const void *y, int y_dtype, int32_t y_count, const float *x0, const void *w, float eps,
+                          void *out, int dtype, int64_t N, int32_t W, void *stream);
+
+/* Whole-projection query / key norm + cache append.  proj [N, ld] holds q (H*D columns at q_col), k (G*D at k_col) and v (G*Dv at
+ * v_col).  q_out [N, H*D] = rms_norm(q) * wq over ALL H*D columns at once; the key is normalised the same way over G*D with wk and
+ * stored at k_cache[slot[n]] ([pool tokens, G*D]); v is stored as it is at v_cache[slot[n]] ([pool tokens, G*Dv]).  slot < 0 skips
+ * the stores. */
+JL_API int jl_qk_norm_append(const void *proj, int dtype, int64_t N, int64_t ld, int32_t q_col, int32_t k_col, int32_t v_col,
+                             int32_t H, int32_t G, int32_t D, int32_t Dv, const void *wq, const void *wk, float eps, void *q_out,
+                             void *k_cache, void *v_cache, const int64_t *slot, void *stream);
+
+/* Attention over the paged pool with a sliding window that keeps the first tokens, a bucketed distance bias and mixed heads:
+ *   visible(i, j) = j <= i and (i - j < window or j < keep_first)
+ *   s_g(i, j) = q_g(i) . k_c(g)(j) * scale + rel[lut[min(i - j, lut_len - 1)], g]          (c(g) = g / (H / G))
+ *   p_g(i, .) = softmax over the visible j;   w_h(i, j) = sum_g talk[h, g] p_g(i, j)  (talk null: w = p)
+ *   out_h(i) = (sum_j w_h(i, j) v_c(h)(j)) * sigmoid(gate_h(i))                             (gate null: no gate)
+ * tiles [n_tiles, 4] int32 = {b, first query position, count (<= TQ), first row}: consecutive rows of one request;
+ * block_tables [*, bt_stride] int32 pages of request b in order; a key j lives at token page * page_size + j % page_size of the
+ * pool.  window <= 0 means no window (plain causal).  rel [rows, H] float and lut int32 may be null (no bias). */
+typedef struct {
+    const void *q; const void *gate; int64_t gate_ld; const void *k_cache; const void *v_cache; void *out;
+    const int32_t *block_tables; const int32_t *tiles; const float *rel; const int32_t *lut; const float *talk;
+    int32_t bt_stride, n_tiles, lut_len, page_size, H, G, D, Dv, window, keep_first, TQ, dtype;
+    float scale;
+} jl_attn_args;
+JL_API int jl_attn_window(const jl_attn_args *a, void *stream);
+/* largest TQ (query rows per tile) the kernel takes for these sizes */
+JL_API int jl_attn_tile_rows(int32_t H, int32_t G, int32_t D, int32_t Dv);
+
+/* Retention (linear attention with a fixed decay per head, no denominator) over the ragged batch, state carried in float:
+ *   q, k rotated (rotate-half pairs on the first rot_dims dimensions, angles from the cos / sin tables [positions, rot_dims/2]),
+ *   k *= D^-1/2;   S_t = decay_h S_(t-1) + k_t v_t^T;   o_t = S_t^T q_t;
+ *   out_h(t) = o_t / sqrt(mean(o_t^2) + eps) * silu(gate_h(t))
+ * proj [N, ld] holds q, k (H*D columns each), v and gate (H*Dv each) at the given columns.  state [slots, H, D, Dv] float: a request
+ * with pos0 == 0 starts from zero (its slot's old content is ignored), otherwise from state[slot]; the final state is written
+ * back.  seq [B, 4] int32 as above. */
+JL_API int jl_retention(const void *proj, int dtype, int64_t ld, int32_t q_col, int32_t k_col, int32_t v_col, int32_t g_col,
+                        const int32_t *seq, int32_t B, int32_t H, int32_t D, int32_t Dv, int32_t rot_dims, const float *cos_t,
+                        const float *sin_t, int64_t table_len, const float *decay, float eps, float *state, void *out,
+                        void *stream);
+
+/* Router of a mixture of experts: s = sigmoid(logits) (float [N, E]); the `top` experts with the largest s + correction are
+ * chosen (ties: lowest index); ids [N, top] int32, weights [N, top] float = s * scale (not renormalised). */
+JL_API int jl_moe_route(const float *logits, const float *correction, int64_t N, int32_t E, int32_t top, float scale, int32_t *ids,
+                        float *weights, void *stream);
+
+/* Rows (token, choice) grouped by expert.  perm [N*top]: sorted row -> flat index n*top + s; offsets [E+1]; tile_expert /
+ * tile_row0 [max_tiles] (max_tiles >= N*top/tile_rows + E): row tiles of at most tile_rows rows of one expert, unused entries -1. */
+JL_API int jl_moe_group(const int32_t *ids, int64_t N, int32_t top, int32_t E, int32_t tile_rows, int32_t *perm, int32_t *offsets,
+                        int32_t *tile_expert, int32_t *tile_row0, int32_t max_tiles, void *stream);
+JL_API int jl_moe_tile_rows(void);
+
+/* Grouped product over the sorted rows: C[r, :] = X[in(r), :] . W[e(r)]^T with W [E, n_out, K].
+ *   mode 0 (up):   in(r) = perm[r] / top;  out[r, :] = relu(C)^2, stored in `dtype` ([N*top, n_out], sorted order)
+ *   mode 1 (down): in(r) = r;              out[perm[r], :] = C * weights[perm[r]], stored as float ([N*top, n_out]) */
+JL_API int jl_moe_gemm(const void *X, const void *Wt, int dtype, int32_t mode, int32_t K, int32_t n_out, int32_t top,
+                       const int32_t *perm, const int32_t *offsets, const int32_t *tile_expert, const int32_t *tile_row0,
+                       int32_t max_tiles, const float *weights, void *out, void *stream);
+
+#ifdef __cplusplus
+}
+#endif
+#endif

@@ -227,3 +227,74 @@ def raise_state_error(code: int, what: str, aux: int = 0):
         raise RuntimeError(f"{what}: fixed capacity exceeded inside the Jacobi state machine (raise max_blocks)")
     if code:
         raise RuntimeError(f"{what}: state machine error {code}")
+
+
+# ---- libjf_layers.so (include/jf_layers.h): layer kernels of the models whose forward is not stock PyTorch ----------------------------
+LAYERS_LIB_PATH = _PKG / "lib" / "libjf_layers.so"
+JL_F32, JL_BF16 = 0, 1
+
+
+class AttnArgs(C.Structure):
+    """jl_attn_args (include/jf_layers.h)."""
+    _fields_ = [("q", _vp), ("gate", _vp), ("gate_ld", _i64), ("k_cache", _vp), ("v_cache", _vp), ("out", _vp),
+                ("block_tables", _vp), ("tiles", _vp), ("rel", _vp), ("lut", _vp), ("talk", _vp),
+                ("bt_stride", _i32), ("n_tiles", _i32), ("lut_len", _i32), ("page_size", _i32), ("H", _i32), ("G", _i32), ("D", _i32),
+                ("Dv", _i32), ("window", _i32), ("keep_first", _i32), ("TQ", _i32), ("dtype", _i32), ("scale", _f32)]
+
+
+_LAYER_SIGNATURES = {
+    "jl_version": (C.c_int, []),
+    "jl_last_error": (C.c_char_p, []),
+    "jl_embed_scale": (C.c_int, [_vp, C.c_int, _vp, _i64, _i32, _f32, _vp, _vp, _vp]),
+    "jl_add_rmsnorm": (C.c_int, [_vp, _vp, C.c_int, _i32, _vp, _vp, _f32, _vp, C.c_int, _i64, _i32, _vp]),
+    "jl_qk_norm_append": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),
+    "jl_attn_window": (C.c_int, [C.POINTER(AttnArgs), _vp]),
+    "jl_attn_tile_rows": (C.c_int, [_i32, _i32, _i32, _i32]),
+    "jl_retention": (C.c_int, [_vp, C.c_int, _i64, _i32, _i32, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _f32,
+                               _vp, _vp, _vp]),
+    "jl_moe_route": (C.c_int, [_vp, _vp, _i64, _i32, _i32, _f32, _vp, _vp, _vp]),
+    "jl_moe_group": (C.c_int, [_vp, _i64, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _vp]),
+    "jl_moe_tile_rows": (C.c_int, []),
+    "jl_moe_gemm": (C.c_int, [_vp, _vp, C.c_int, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
+}
+LAYER_SYMBOLS = tuple(_LAYER_SIGNATURES)
+_LAYERS = None
+
+
+def layers():
+    """The layer-kernel library.  Loads what is built; compiles it (hipcc, about a minute) only when there is none — a fresh
+    checkout's first call.  There is no CPU or eager fallback for these kernels either."""
+    global _LAYERS
+    if _LAYERS is None:
+        p = Path(os.environ.get("JF_LAYERS_LIB", LAYERS_LIB_PATH))
+        if not p.exists():
+            if "JF_LAYERS_LIB" in os.environ:
+                raise NativeLibraryError(f"{p} not found")
+            from . import _build
+            try:
+                _build.build_layers()
+            except Exception as e:
+                raise NativeLibraryError(f"cannot build {p}: {e}") from e
+        try:
+            lib_ = C.CDLL(str(p))
+        except OSError as e:
+            raise NativeLibraryError(f"cannot load {p}: {e}") from e
+        for name, (res, args) in _LAYER_SIGNATURES.items():
+            try:
+                fn = getattr(lib_, name)
+            except AttributeError as e:
+                raise NativeLibraryError(f"{p} does not export {name}") from e
+            fn.restype, fn.argtypes = res, args
+        _LAYERS = lib_
+    return _LAYERS
+
+
+def check_layers(rc: int, what: str = ""):
+    if rc == 0:
+        return
+    msg = layers().jl_last_error()
+    msg = msg.decode() if isinstance(msg, (bytes, bytearray)) else str(msg)
+    text = f"{what}: {msg}" if what else msg
+    if rc == -1:
+        raise ValueError(text)
+    raise RuntimeError(text)

@@ -1,0 +1,40 @@
+"""Storage behind the ragged step: a pool of key/value pages per attention layer run and a table of recurrent-state slots per
+recurrent layer run.  Which page or slot a request uses is bookkeeping elsewhere (``BlockManager`` hands out page ids, the
+runner hands out slots); this class only owns the memory, sized once.
+
+A *layer run* is one execution of a layer in a forward: a model that repeats a span of layers with the same weights has one
+run — and therefore one cache or state of its own — per repetition."""
+from __future__ import annotations
+
+from dataclasses import dataclass
+from typing import List, Optional
+
+import torch
+
+
+@dataclass
+class RunSpec:
+    """Memory one layer run needs.  kind "kv": ``k_width`` / ``v_width`` elements per cached token (all key/value heads side by
+    side).  kind "state": a float tensor of ``state_shape`` per slot.  kind None: nothing."""
+    kind: Optional[str]
+    k_width: int = 0
+    v_width: int = 0
+    state_shape: tuple = ()
+
+
+class PagedStateCache:
+    def __init__(self, specs: List[RunSpec], num_pages: int, page_size: int, num_slots: int, device, dtype):
+        self.num_pages, self.page_size, self.num_slots = int(num_pages), int(page_size), int(num_slots)
+        self.P = self.num_slots                      # a live request owns one slot: the scheduler's admission limit
+        tokens = self.num_pages * self.page_size
+        self.k: List[Optional[torch.Tensor]] = []
+        self.v: List[Optional[torch.Tensor]] = []
+        self.state: List[Optional[torch.Tensor]] = []
+        for s in specs:
+            kv = s.kind == "kv"
+            self.k.append(torch.zeros((tokens, s.k_width), dtype=dtype, device=device) if kv else None)
+            self.v.append(torch.zeros((tokens, s.v_width), dtype=dtype, device=device) if kv else None)
+            self.state.append(torch.zeros((self.num_slots, *s.state_shape), dtype=torch.float32, device=device) if s.kind == "state" else None)
+
+    def bytes(self) -> int:
+        return sum(t.numel() * t.element_size() for ts in (self.k, self.v, self.state) for t in ts if t is not None)

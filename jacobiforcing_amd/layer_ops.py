@@ -1,0 +1,239 @@
+"""torch-facing wrappers over ``libjf_layers.so`` (include/jf_layers.h): torch allocates and owns the memory, every operation
+runs in the HIP library.  Shapes are checked here, on the host, before a launch.
+
+A step's tokens form one ragged batch (``RaggedBatch``): N token rows, the rows of a request consecutive, with the per-request
+records and tiles the kernels read."""
+from __future__ import annotations
+
+import ctypes as C
+from dataclasses import dataclass
+from typing import List, Optional, Sequence, Tuple
+
+import numpy as np
+import torch
+
+from . import _native as N
+
+
+def _ptr(t: Optional[torch.Tensor]):
+    return None if t is None else C.c_void_p(t.data_ptr())
+
+
+def _stream(device: torch.device):
+    return C.c_void_p(torch.cuda.current_stream(device).cuda_stream) if device.type == "cuda" else None
+
+
+def _code(dt: torch.dtype) -> int:
+    if dt == torch.float32:
+        return N.JL_F32
+    if dt == torch.bfloat16:
+        return N.JL_BF16
+    raise ValueError(f"activations must be float32 or bfloat16, got {dt}")
+
+
+def _need(cond: bool, msg: str) -> None:
+    if not cond:
+        raise ValueError(msg)
+
+
+def _dev(t: torch.Tensor) -> None:
+    if t.device.type != "cuda":
+        raise N.NativeLibraryError("the layer kernels run on the GPU only (no CPU fallback)")
+
+
+@dataclass
+class RaggedBatch:
+    """What one step runs: requests b = 0..B-1 with ``counts[b]`` new tokens from position ``starts[b]``, state slot ``slots[b]``
+    and pages ``block_tables[b]``.  Device tensors: ``seq`` [B, 4] int32 {row0, count, pos0, slot}, ``kv_slot`` [N] int64 (pool
+    token of every new row), ``tables`` [B, C] int32."""
+    B: int
+    N: int
+    counts: List[int]
+    starts: List[int]
+    seq: torch.Tensor
+    kv_slot: torch.Tensor
+    tables: torch.Tensor
+    page_size: int
+    max_pos: int
+    max_page: int
+    max_slot: int
+    _tiles: dict
+
+    @classmethod
+    def build(cls, counts: Sequence[int], starts: Sequence[int], slots: Sequence[int], block_tables: Sequence[Sequence[int]],
+              page_size: int, device) -> "RaggedBatch":
+        B = len(counts)
+        row0 = np.concatenate([[0], np.cumsum(counts)]).astype(np.int64)
+        seq = np.stack([row0[:-1], np.asarray(counts), np.asarray(starts), np.asarray(slots)], 1).astype(np.int32).reshape(B, 4)
+        C_ = max(1, max(len(t) for t in block_tables))
+        bt = np.full((B, C_), -1, dtype=np.int32)
+        kv = np.empty(int(row0[-1]), dtype=np.int64)
+        for b in range(B):
+            t = np.asarray(block_tables[b], dtype=np.int64)
+            bt[b, :t.size] = t
+            pos = starts[b] + np.arange(counts[b], dtype=np.int64)
+            if counts[b] and (starts[b] + counts[b] + page_size - 1) // page_size > t.size:
+                raise ValueError(f"request {b}: {t.size} pages do not hold {starts[b] + counts[b]} tokens")
+            kv[row0[b]:row0[b + 1]] = t[pos // page_size] * page_size + pos % page_size
+        dev = torch.device(device)
+        return cls(B=B, N=int(row0[-1]), counts=list(map(int, counts)), starts=list(map(int, starts)),
+                   seq=torch.from_numpy(seq).to(dev), kv_slot=torch.from_numpy(kv).to(dev), tables=torch.from_numpy(bt).to(dev),
+                   page_size=int(page_size), max_pos=max(int(s) + int(c) for s, c in zip(starts, counts)), max_page=int(bt.max()),
+                   max_slot=int(max(slots)), _tiles={})
+
+    def tiles(self, tq: int) -> torch.Tensor:
+        """[n_tiles, 4] int32 {b, first query position, count, first row}: each request's rows cut into runs of at most ``tq``."""
+        t = self._tiles.get(tq)
+        if t is None:
+            rows, r0 = [], 0
+            for b, (c, s) in enumerate(zip(self.counts, self.starts)):
+                for o in range(0, c, tq):
+                    rows.append((b, s + o, min(tq, c - o), r0 + o))
+                r0 += c
+            t = self._tiles[tq] = torch.tensor(rows, dtype=torch.int32, device=self.seq.device).reshape(-1, 4)
+        return t
+
+
+def embed_scale(embed: torch.Tensor, ids: torch.Tensor, scale: float, want_copy: bool) -> Tuple[torch.Tensor, Optional[torch.Tensor]]:
+    _dev(embed)
+    _need(embed.dim() == 2 and embed.is_contiguous() and ids.dtype == torch.int64 and ids.is_contiguous(), "embed_scale: embed [V, W], ids int64 [N]")
+    n, W = ids.numel(), embed.shape[1]
+    x = torch.empty((n, W), dtype=torch.float32, device=embed.device)
+    x0 = torch.empty_like(x) if want_copy else None
+    N.check_layers(N.layers().jl_embed_scale(_ptr(embed), _code(embed.dtype), _ptr(ids), n, W, float(scale), _ptr(x), _ptr(x0),
+                                            _stream(embed.device)), "jl_embed_scale")
+    return x, x0
+
+
+def add_rmsnorm(x: torch.Tensor, y: Optional[torch.Tensor], x0: Optional[torch.Tensor], w: Optional[torch.Tensor], eps: float,
+                out_dtype: Optional[torch.dtype]) -> Optional[torch.Tensor]:
+    """x (float [N, W], in place) += y summed over its middle axis ([N, W] or [N, S, W], float or bf16) + x0; returns
+    rms_norm(x) * w in ``out_dtype`` (None: the update only)."""
+    _dev(x)
+    n, W = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous(), "add_rmsnorm: x must be contiguous float32 [N, W]")
+    cnt = 0
+    if y is not None:
+        _need(y.is_contiguous() and y.shape[0] == n and y.shape[-1] == W and y.dim() in (2, 3), "add_rmsnorm: y must be [N, W] or [N, S, W]")
+        cnt = 1 if y.dim() == 2 else y.shape[1]
+    if x0 is not None:
+        _need(x0.shape == x.shape and x0.dtype == torch.float32 and x0.is_contiguous(), "add_rmsnorm: x0 must match x")
+    out = None
+    if out_dtype is not None:
+        out = torch.empty((n, W), dtype=out_dtype, device=x.device)
+        if w is not None:
+            _need(w.dtype == out_dtype and w.numel() == W and w.is_contiguous(), "add_rmsnorm: the weight has the output's dtype and W entries")
+    N.check_layers(N.layers().jl_add_rmsnorm(_ptr(x), _ptr(y), _code(y.dtype) if y is not None else 0, cnt, _ptr(x0), _ptr(w), float(eps),
+                                            _ptr(out), _code(out_dtype or torch.float32), n, W, _stream(x.device)), "jl_add_rmsnorm")
+    return out
+
+
+def qk_norm_append(proj: torch.Tensor, cols: Tuple[int, int, int], H: int, G: int, D: int, Dv: int, wq: torch.Tensor, wk: torch.Tensor,
+                   eps: float, k_cache: torch.Tensor, v_cache: torch.Tensor, kv_slot: torch.Tensor) -> torch.Tensor:
+    _dev(proj)
+    n, ld = proj.shape
+    dt = proj.dtype
+    _need(proj.is_contiguous() and kv_slot.dtype == torch.int64 and kv_slot.numel() == n, "qk_norm_append: proj [N, ld], one pool token per row")
+    _need(wq.numel() == H * D and wk.numel() == G * D and wq.dtype == dt and wk.dtype == dt, "qk_norm_append: norm weights over the whole projections")
+    _need(k_cache.dtype == dt and v_cache.dtype == dt and k_cache.is_contiguous() and v_cache.is_contiguous() and
+          k_cache.shape[-1] == G * D and v_cache.shape[-1] == G * Dv and k_cache.shape[0] == v_cache.shape[0], "qk_norm_append: pools [tokens, G*D] / [tokens, G*Dv]")
+    q = torch.empty((n, H * D), dtype=dt, device=proj.device)
+    N.check_layers(N.layers().jl_qk_norm_append(_ptr(proj), _code(dt), n, ld, cols[0], cols[1], cols[2], H, G, D, Dv, _ptr(wq), _ptr(wk), float(eps),
+                                               _ptr(q), _ptr(k_cache), _ptr(v_cache), _ptr(kv_slot), _stream(proj.device)), "jl_qk_norm_append")
+    return q
+
+
+def attn_tile_rows(H: int, G: int, D: int, Dv: int) -> int:
+    tq = int(N.layers().jl_attn_tile_rows(H, G, D, Dv))
+    if tq <= 0:
+        raise ValueError(f"attention sizes heads={H} kv_heads={G} dim={D} vdim={Dv} exceed the kernel's tile")
+    return tq
+
+
+def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor, batch: RaggedBatch,
+                H: int, G: int, D: int, Dv: int, scale: float, window: int, keep_first: int, rel: Optional[torch.Tensor],
+                lut: Optional[torch.Tensor], talk: Optional[torch.Tensor]) -> torch.Tensor:
+    """q [N, H*D]; gate a [N, H*Dv] view (column range of the projection output, row stride free) or None.  Returns [N, H*Dv]."""
+    _dev(q)
+    dt = q.dtype
+    n = q.shape[0]
+    _need(q.is_contiguous() and q.shape[1] == H * D and n == batch.N, "attn_window: q [N, H*D] of the batch")
+    _need(k_cache.dtype == dt and v_cache.dtype == dt and k_cache.shape[-1] == G * D and v_cache.shape[-1] == G * Dv, "attn_window: pool dtype / widths")
+    pool_tokens = k_cache.shape[0]
+    _need(pool_tokens % batch.page_size == 0 and batch.max_page < pool_tokens // batch.page_size, "attn_window: a page lies outside the pool")
+    if gate is not None:
+        _need(gate.shape == (n, H * Dv) and gate.stride(1) == 1 and gate.dtype == dt, "attn_window: gate [N, H*Dv]")
+    for t, shape in ((rel, None), (talk, (H, H))):
+        if t is not None:
+            _need(t.dtype == torch.float32 and t.is_contiguous() and (shape is None or tuple(t.shape) == shape), "attn_window: float tables")
+    if rel is not None:
+        _need(lut is not None and lut.dtype == torch.int32 and rel.shape[1] == H, "attn_window: rel [rows, H] with its lut")
+    tq = attn_tile_rows(H, G, D, Dv)
+    tiles = batch.tiles(tq)
+    out = torch.empty((n, H * Dv), dtype=dt, device=q.device)
+    a = N.AttnArgs(q=q.data_ptr(), gate=gate.data_ptr() if gate is not None else None, gate_ld=gate.stride(0) if gate is not None else 0,
+                   k_cache=k_cache.data_ptr(), v_cache=v_cache.data_ptr(), out=out.data_ptr(), block_tables=batch.tables.data_ptr(),
+                   tiles=tiles.data_ptr(), rel=rel.data_ptr() if rel is not None else None, lut=lut.data_ptr() if rel is not None else None,
+                   talk=talk.data_ptr() if talk is not None else None, bt_stride=batch.tables.shape[1], n_tiles=tiles.shape[0],
+                   lut_len=lut.numel() if rel is not None else 0, page_size=batch.page_size, H=H, G=G, D=D, Dv=Dv, window=int(window),
+                   keep_first=int(keep_first), TQ=tq, dtype=_code(dt), scale=float(scale))
+    N.check_layers(N.layers().jl_attn_window(C.byref(a), _stream(q.device)), "jl_attn_window")
+    return out
+
+
+def retention(proj: torch.Tensor, cols: Tuple[int, int, int, int], batch: RaggedBatch, H: int, D: int, Dv: int, rot_dims: int,
+              cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], decay: torch.Tensor, eps: float, state: torch.Tensor) -> torch.Tensor:
+    """proj [N, ld] with q, k, v, gate at ``cols``; state [slots, H, D, Dv] float (updated in place).  Returns [N, H*Dv]."""
+    _dev(proj)
+    n, ld = proj.shape
+    _need(proj.is_contiguous() and n == batch.N, "retention: proj [N, ld] of the batch")
+    _need(state.dtype == torch.float32 and state.is_contiguous() and tuple(state.shape[1:]) == (H, D, Dv), "retention: state [slots, H, D, Dv] float")
+    _need(batch.max_slot < state.shape[0], "retention: a slot lies outside the state")
+    _need(decay.dtype == torch.float32 and decay.numel() == H, "retention: one decay per head")
+    _need(max(cols[0], cols[1]) + H * D <= ld and max(cols[2], cols[3]) + H * Dv <= ld, "retention: columns do not fit the row")
+    tl = 0
+    if rot_dims:
+        _need(cos is not None and cos.dtype == torch.float32 and cos.is_contiguous() and cos.shape == sin.shape and cos.shape[1] == rot_dims // 2,
+              "retention: cos / sin [positions, rot_dims / 2] float")
+        tl = cos.shape[0]
+        _need(batch.max_pos <= tl, "retention: the angle tables are shorter than the batch's positions")
+    out = torch.empty((n, H * Dv), dtype=proj.dtype, device=proj.device)
+    N.check_layers(N.layers().jl_retention(_ptr(proj), _code(proj.dtype), ld, cols[0], cols[1], cols[2], cols[3], _ptr(batch.seq), batch.B, H, D, Dv,
+                                          rot_dims, _ptr(cos), _ptr(sin), tl, _ptr(decay), float(eps), _ptr(state), _ptr(out),
+                                          _stream(proj.device)), "jl_retention")
+    return out
+
+
+def moe_experts(h: torch.Tensor, router_logits: torch.Tensor, correction: Optional[torch.Tensor], top: int, scale: float,
+                w_up: torch.Tensor, w_down: torch.Tensor) -> torch.Tensor:
+    """Routed experts down(relu(up h)^2): h [N, W], router_logits float [N, E], w_up [E, ff, W], w_down [E, W, ff].  Returns the
+    weighted expert outputs per choice, float [N, top, W] (their sum over the middle axis is the layer's output)."""
+    _dev(h)
+    n, W = h.shape
+    E, ff = w_up.shape[0], w_up.shape[1]
+    dev, dt = h.device, h.dtype
+    _need(h.is_contiguous() and router_logits.dtype == torch.float32 and router_logits.is_contiguous() and tuple(router_logits.shape) == (n, E),
+          "moe_experts: h [N, W], logits float [N, E]")
+    _need(tuple(w_up.shape) == (E, ff, W) and tuple(w_down.shape) == (E, W, ff) and w_up.dtype == dt and w_down.dtype == dt and
+          w_up.is_contiguous() and w_down.is_contiguous(), "moe_experts: expert weights [E, ff, W] / [E, W, ff] in the activation dtype")
+    if correction is not None:
+        _need(correction.dtype == torch.float32 and correction.numel() == E, "moe_experts: correction float [E]")
+    L, st = N.layers(), _stream(dev)
+    ids = torch.empty((n, top), dtype=torch.int32, device=dev)
+    wts = torch.empty((n, top), dtype=torch.float32, device=dev)
+    N.check_layers(L.jl_moe_route(_ptr(router_logits), _ptr(correction), n, E, top, float(scale), _ptr(ids), _ptr(wts), st), "jl_moe_route")
+    tm = int(L.jl_moe_tile_rows())
+    rows = n * top
+    max_tiles = rows // tm + E
+    perm = torch.empty((rows,), dtype=torch.int32, device=dev)
+    offsets = torch.empty((E + 1,), dtype=torch.int32, device=dev)
+    tile_e = torch.empty((max_tiles,), dtype=torch.int32, device=dev)
+    tile_r = torch.empty((max_tiles,), dtype=torch.int32, device=dev)
+    N.check_layers(L.jl_moe_group(_ptr(ids), n, top, E, tm, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles, st), "jl_moe_group")
+    act = torch.empty((rows, ff), dtype=dt, device=dev)
+    N.check_layers(L.jl_moe_gemm(_ptr(h), _ptr(w_up), _code(dt), 0, W, ff, top, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles,
+                                 None, _ptr(act), st), "jl_moe_gemm(up)")
+    y = torch.empty((n, top, W), dtype=torch.float32, device=dev)
+    N.check_layers(L.jl_moe_gemm(_ptr(act), _ptr(w_down), _code(dt), 1, ff, W, top, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles,
+                                 _ptr(wts), _ptr(y), st), "jl_moe_gemm(down)")
+    return y
