@@ -20,6 +20,8 @@ _FIELDS = [
     # "contiguous": one static cache row per request (this package's layout); "paged": the reference's pool of blocks addressed
     # through block tables and slot mappings (layers/attention.py:10-40, MR:1204-1265) — same decodes, for callers that want its memory model
     ("kv_cache_layout", str, "contiguous"),
+    # "auto": bfloat16 on the GPU (float32 on the CPU); "bfloat16" / "float32" force it.  float32 = every product in true 32-bit
+    ("dtype", str, "auto"),
     # Jacobi defaults of the engine (requests override them through SamplingParams)
     ("jacobi_enabled", bool, True), ("jacobi_block_len", int, 64), ("jacobi_max_blocks", int, 2),
     ("jacobi_spawn_ratio", float, 0.8), ("jacobi_lookahead_start_ratio", float, 0.0),
@@ -41,7 +43,8 @@ def _resolve_model_dir(model: str) -> Path:
 
 def _finish_init(self) -> None:
     model_dir = _resolve_model_dir(self.model)
-    assert self.kvcache_block_size % 256 == 0
+    # pages of 256 tokens for the padded families (the reference's check); a ragged family's pool may use pages of 64
+    assert self.kvcache_block_size % 64 == 0
     assert 1 <= self.tensor_parallel_size <= 8
     if self.kv_cache_layout not in ("contiguous", "paged"):
         raise ValueError(f"kv_cache_layout must be 'contiguous' or 'paged', got {self.kv_cache_layout!r}")
@@ -49,8 +52,12 @@ def _finish_init(self) -> None:
         raise NotImplementedError("tensor parallelism is not part of this path: prompts replicate across GPUs "
                                   "(one process per GPU); use tensor_parallel_size=1")
     self.model_path = str(model_dir)
-    from .modeling.qwen2 import Qwen2Config
-    self.hf_config = Qwen2Config.from_json(model_dir / "config.json")
+    from .modeling import family_of, read_model_config
+    self.hf_config = read_model_config(model_dir)
+    if family_of(self.hf_config) != "ragged":
+        assert self.kvcache_block_size % 256 == 0
+    if self.dtype not in ("auto", "bfloat16", "float32"):
+        raise ValueError(f"dtype must be 'auto', 'bfloat16' or 'float32', got {self.dtype!r}")
     self.max_model_len = min(self.max_model_len, self.hf_config.max_position_embeddings)
     assert self.max_num_batched_tokens >= self.max_model_len
 

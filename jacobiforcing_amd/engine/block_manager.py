@@ -68,6 +68,17 @@ class BlockManager:
         seq.num_cached_tokens = 0
         seq.num_permanent_spec_blocks = 0
 
+    def ensure(self, seq: Sequence, num_tokens: int) -> bool:
+        """The ragged step's allocation: grow ``seq``'s table until it holds ``num_tokens`` positions.  All or nothing: False (and
+        no change) when the free pages do not suffice.  Pages are taken from the head of the free list, like every other grow."""
+        need = -(-int(num_tokens) // self.block_size) - len(seq.block_table)
+        if need > len(self.free_block_ids):
+            return False
+        for _ in range(max(need, 0)):
+            self._grow(seq)
+            seq.block_table_version += 1
+        return True
+
     def can_append(self, seq: Sequence) -> bool:
         opens_block = len(seq) % self.block_size == 1
         return len(self.free_block_ids) >= int(opens_block)

@@ -56,7 +56,50 @@ class LLMEngine:
         seq = Sequence(prompt, sampling_params)
         self.scheduler.add(seq)
 
+    # ---- ragged model families: every step is one mixed batch ------------------------------------------------------------------
+    def _step_ragged(self):
+        items = self.scheduler.schedule_ragged()
+        logits, owners = self.model_runner.run_ragged(items)
+        self.scheduler.postprocess(owners, self.model_runner.sample(logits, owners) if owners else [])
+        outputs = []
+        for seq in owners:
+            if seq.is_finished:
+                outputs.append((seq.seq_id, seq.completion_token_ids))
+                self.model_runner.release(seq)
+        prompt_tokens = sum(n for _, n in items if n > 1)
+        return outputs, (prompt_tokens if prompt_tokens else -len(owners))
+
+    def replay_step(self, entries, end=()):
+        """Run one step of a GIVEN schedule through the engine's own step function, cache and bookkeeping, sampling nothing.
+        ``entries`` = [(request key, its next tokens, places among them whose logits are wanted)]; a key seen for the first time
+        is admitted (a state slot; pages as its tokens arrive), a request may skip steps, and the requests in ``end`` give pages
+        and slot back after the step.  Returns float logits [wanted, vocab] in the order of the entries and their places."""
+        if not self.model_runner.ragged:
+            raise NotImplementedError("replaying a schedule needs a ragged model family (mixed batches of portions and single tokens)")
+        live = self.__dict__.setdefault("_replay_live", {})
+        items, want = [], []
+        for key, tokens, places in entries:
+            seq = live.get(key)
+            if seq is None:
+                seq = live[key] = Sequence(list(tokens), SamplingParams(temperature=0.0, max_tokens=1 << 30, ignore_eos=True))
+                self.scheduler.admit(seq)
+            else:
+                seq.extend_tokens(tokens)
+            self.scheduler.reserve(seq, len(tokens))
+            items.append((seq, len(tokens)))
+            want.append(list(places))
+        logits = None
+        if items:
+            logits, _ = self.model_runner.run_ragged(items, want)
+        for key in end:
+            seq = live.pop(key, None)
+            if seq is not None:
+                self.scheduler.finish(seq)
+        return logits
+
     def step(self):
+        if self.model_runner.ragged:
+            return self._step_ragged()
         seqs, is_prefill = self.scheduler.schedule()
         result = self.model_runner.call("run", seqs, is_prefill)
         if result is None or (is_prefill and len(result) > 0 and result[0] == []):              # ENG:90-93

@@ -20,6 +20,8 @@ import torch
 
 from .. import _native, ops
 from ..config import Config
+from .. import layer_ops
+from ..modeling import MODEL_REGISTRY, architecture_of, family_of
 from ..modeling.qwen2 import Qwen2Model, Qwen2Weights, StaticKVCache
 from .jacobi_decoding import JacobiDecoder
 from .jacobi_decoding_nongreedy import JacobiDecoderNonGreedy
@@ -173,12 +175,20 @@ class ModelRunner:
         self.rank, self.world_size = 0, 1
         dev = device or os.environ.get("JF_DEVICE") or ("cuda" if torch.cuda.is_available() else "cpu")
         self.device = torch.device(dev)
-        if self.device.type == "cuda":
+        if self.device.type == "cuda" and family_of(config.hf_config) != "ragged":
             _native.lib()                                     # fail loudly when the HIP extension is missing
         hf = config.hf_config
         dtype = torch.bfloat16 if self.device.type == "cuda" else torch.float32
+        if getattr(config, "dtype", "auto") != "auto":
+            dtype = getattr(torch, config.dtype)
         if os.environ.get("JF_DTYPE"):
             dtype = getattr(torch, os.environ["JF_DTYPE"])
+        self.ragged = family_of(hf) == "ragged"
+        self.profiler = ProfileTimer(self.device)
+        self.block_manager = None
+        if self.ragged:
+            self._init_ragged(config, dtype)
+            return
         sw = ModelRunner.shared_weights
         if sw is not None and sw.embed.device == self.device and tuple(sw.embed.shape) == (hf.vocab_size, hf.hidden_size) \
                 and len(sw.layers) == hf.num_hidden_layers:
@@ -208,12 +218,68 @@ class ModelRunner:
         else:
             self.kv_cache = StaticKVCache(hf, self.max_rows, config.max_model_len, 0, 1, self.device, dtype=dtype)
         self.free_rows = list(range(self.max_rows))
-        self.block_manager = None
         self.jacobi_decoder = None
         self._mb_decoders = {}
-        self.profiler = ProfileTimer(self.device)
         self._kv_host = [0] * self.max_rows
         self._logit_idx = {}
+
+    # ---- ragged model families: one flat batch over a paged pool + state slots -----------------------------------------------
+    def _init_ragged(self, config: Config, dtype) -> None:
+        """Model, pool and slots of a ragged family.  The layer kernels have no CPU form: a missing library or a CPU device is an
+        error here, not a fallback.  Slots = ``max_num_seqs`` (at most JF_MAX_ROWS); pages = ``num_kvcache_blocks`` when given,
+        else what ``max_model_len`` tokens per slot need."""
+        import importlib
+        if self.device.type != "cuda":
+            raise _native.NativeLibraryError("ragged model families run on the GPU only (their layer kernels have no CPU form)")
+        _native.layers()
+        hf = config.hf_config
+        mod = importlib.import_module(MODEL_REGISTRY[architecture_of(config.model_path)][0])
+        has = bool(list(Path(config.model_path).glob("*.safetensors")))
+        if has:
+            _, self.model = mod.load_model_directory(config.model_path, self.device, dtype, max_positions=config.max_model_len)
+        else:
+            import sys
+            print(f"[ModelRunner] no *.safetensors under {config.model_path}: using random-init weights", file=sys.stderr, flush=True)
+            self.model = mod.random_model(hf, self.device, dtype, max_positions=config.max_model_len,
+                                          seed=int(os.environ.get("JF_WEIGHT_SEED", "0")))
+        self.weights = self.model.w
+        self.block_size = config.kvcache_block_size
+        self.max_rows = int(min(config.max_num_seqs, int(os.environ.get("JF_MAX_ROWS", "64"))))
+        if config.num_kvcache_blocks <= 0:
+            config.num_kvcache_blocks = self.max_rows * (-(-config.max_model_len // self.block_size))
+        self.paged = True
+        self.kv_cache = self.model.new_cache(config.num_kvcache_blocks, self.block_size, self.max_rows)
+        self.free_rows = list(range(self.max_rows))
+        self.jacobi_decoder, self._mb_decoders = None, {}
+
+    @torch.inference_mode()
+    def run_ragged(self, items, want=None):
+        """The ragged families' step function.  ``items`` = [(request, count)]: each request's next ``count`` tokens
+        (``token_ids[num_cached_tokens:][:count]``) run as one flat batch from the cache and state earlier steps left; pages come
+        from the request's block table, the state slot is its cache row.  ``want[i]`` lists the places among request i's tokens
+        whose logits are returned (default: the last one when the step reaches the end of what the request holds — the position
+        a sampler continues from).  Returns (float logits [wanted, vocab], the request of every returned row)."""
+        counts, starts, slots, tables, ids, rows, owners, r0 = [], [], [], [], [], [], [], 0
+        for i, (seq, n) in enumerate(items):
+            s0 = seq.num_cached_tokens
+            if n <= 0 or s0 + n > len(seq):
+                raise ValueError(f"request {seq.seq_id}: {n} tokens from {s0} of {len(seq)}")
+            if s0 + n > self.config.max_model_len:
+                raise RuntimeError(f"Sequence needs {s0 + n} positions but max_model_len={self.config.max_model_len}")
+            w = want[i] if want is not None else ([n - 1] if s0 + n == len(seq) else [])
+            if any(not 0 <= k < n for k in w):
+                raise ValueError(f"request {seq.seq_id}: wanted places {w} outside its {n} tokens")
+            counts.append(n); starts.append(s0); slots.append(self._row(seq)); tables.append(seq.block_table)
+            ids += seq.token_ids[s0:s0 + n]
+            rows += [r0 + k for k in w]
+            owners += [seq] * len(w)
+            r0 += n
+        batch = layer_ops.RaggedBatch.build(counts, starts, slots, tables, self.block_size, self.device)
+        dev_ids = torch.tensor(ids, dtype=torch.int64, device=self.device)
+        logits = self.model.forward(dev_ids, batch, self.kv_cache, torch.tensor(rows, dtype=torch.int64, device=self.device))
+        for seq, n in items:
+            seq.num_cached_tokens += n
+        return logits, owners
 
     # ------------------------------------------------------------------------------------------
     def call(self, method_name, *args):
@@ -477,6 +543,11 @@ class ModelRunner:
             logits = self._forward_rows(seqs, ids, [len(seq) - 1 for seq in seqs], [1] * len(seqs))
         for seq in seqs:
             seq.num_cached_tokens = len(seq)
+        return self.sample(logits, seqs)
+
+    def sample(self, logits: torch.Tensor, seqs: List[Sequence]):
+        """One token per row of ``logits`` for the request it belongs to: argmax at temperature 0, else Gumbel-max over the
+        (filtered) softmax."""
         temps = [float(seq.temperature) for seq in seqs]
         if all(t == 0.0 for t in temps):
             return [int(t) for t in ops.argmax_rows(logits).cpu().tolist()]

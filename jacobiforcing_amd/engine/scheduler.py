@@ -81,6 +81,62 @@ class Scheduler:
         self.running.extendleft(reversed(batch))
         return batch
 
+    # ---- ragged step: prompt portions and decoded tokens in one batch ----------------------------------------------------------
+    def schedule_ragged(self) -> List[Tuple[Sequence, int]]:
+        """One step's work for a ragged model family as (request, number of its next tokens).  Every running request continues —
+        the next portion of its prompt while tokens of it are uncached, else its one new token — within the step's token budget
+        (``max_num_batched_tokens``); then waiting requests are admitted while a state slot, pages and budget last.  When the
+        pages run out, the newest running request is preempted (it gives pages and slot back and is prefilled again later)."""
+        bm, budget, items = self.block_manager, self.max_num_batched_tokens, []
+        for seq in list(self.running):
+            if seq not in self.running:                        # preempted below
+                continue
+            if budget <= 0 or len(items) >= self.max_num_seqs:
+                break
+            n = min(len(seq) - seq.num_cached_tokens, budget)
+            while n > 0 and not bm.ensure(seq, seq.num_cached_tokens + n):
+                victim = self.running[-1]
+                self.preempt(victim)
+                self.running.remove(victim)
+                items = [it for it in items if it[0] is not victim]
+                if victim is seq:
+                    n = 0
+            if n > 0:
+                items.append((seq, n))
+                budget -= n
+        while self.waiting and budget > 0 and len(items) < self.max_num_seqs:
+            seq = self.waiting[0]
+            if self.row_capacity is not None and len(self.running) >= self.row_capacity:
+                break
+            n = min(len(seq) - seq.num_cached_tokens, budget)
+            if not bm.ensure(seq, seq.num_cached_tokens + n):
+                break
+            self.admit(self.waiting.popleft())
+            items.append((seq, n))
+            budget -= n
+        if not items and (self.waiting or self.running):
+            raise RuntimeError("the page pool cannot hold a single request's next tokens (raise num_kvcache_blocks)")
+        return items
+
+    def admit(self, seq: Sequence) -> None:
+        """Make ``seq`` a running request (the ragged scheduler above, or a caller that replays a given schedule)."""
+        if self.row_capacity is not None and len(self.running) >= self.row_capacity:
+            raise RuntimeError(f"all {self.row_capacity} state slots are taken")
+        seq.status = SequenceStatus.RUNNING
+        self.running.append(seq)
+
+    def reserve(self, seq: Sequence, count: int) -> None:
+        """Pages for ``count`` more tokens of a running request, or an error: a replayed schedule is not rearranged."""
+        if not self.block_manager.ensure(seq, seq.num_cached_tokens + count):
+            raise RuntimeError(f"no free pages for {count} more tokens of request {seq.seq_id} ({len(self.block_manager.free_block_ids)} "
+                               f"pages of {self.block_manager.block_size} free)")
+
+    def finish(self, seq: Sequence) -> None:
+        """End a running request: its pages go back to the pool, its slot to the runner."""
+        self._finish(seq)
+        if self.release_row is not None:
+            self.release_row(seq)
+
     def preempt(self, seq: Sequence) -> None:
         """Back to the queue (SCH:70-73).  The request also gives its cache row back — it is re-prefilled from scratch when it
         is admitted again — so that the admission limit above counts rows that are really free."""

@@ -281,3 +281,7 @@ class LokizenModel:
 def load_model_directory(model_dir, device, dtype=torch.bfloat16, max_positions: int = 8192):
     cfg = LokizenConfig.from_json(Path(model_dir) / "config.json")
     return cfg, LokizenModel(cfg, LokizenWeights.from_safetensors(cfg, model_dir, device, dtype), max_positions)
+
+
+def random_model(cfg: LokizenConfig, device, dtype=torch.bfloat16, max_positions: int = 8192, seed: int = 0) -> LokizenModel:
+    return LokizenModel(cfg, LokizenWeights.random(cfg, device, dtype, seed), max_positions)
