@@ -158,14 +158,15 @@ def random_tensors(cfg: LokizenConfig, seed: int = 0, rel_rows: int = 16) -> Dic
     W = cfg.hidden_size
     rnd = lambda *s, std=1.0: (torch.randn(*s, generator=g) * std).to(torch.bfloat16).float()
     lin = lambda o, i: rnd(o, i, std=i ** -0.5)
-    t = {"embed": rnd(cfg.vocab_size, W), "final.norm": 1 + rnd(W, std=0.1), "head": lin(cfg.vocab_size, W)}
+    one = lambda n: (1 + torch.randn(n, generator=g) * 0.1).to(torch.bfloat16).float()
+    t = {"embed": rnd(cfg.vocab_size, W), "final.norm": one(W), "head": lin(cfg.vocab_size, W)}
     for i, L in enumerate(cfg.layers):
         p, m = f"l{i}.", L["mixer"]
-        t[p + "norm1"] = 1 + rnd(W, std=0.1)
+        t[p + "norm1"] = one(W)
         if L["type"] == "attention":
             H, G, D, Dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
             t.update({p + "mix.q": lin(H * D, W), p + "mix.k": lin(G * D, W), p + "mix.v": lin(G * Dv, W), p + "mix.g": lin(H * Dv, W),
-                      p + "mix.o": lin(W, H * Dv), p + "mix.q.norm": 1 + rnd(H * D, std=0.1), p + "mix.k.norm": 1 + rnd(G * D, std=0.1),
+                      p + "mix.o": lin(W, H * Dv), p + "mix.q.norm": one(H * D), p + "mix.k.norm": one(G * D),
                       p + "mix.rel": rnd(rel_rows, H), p + "mix.talk": (torch.eye(H) + rnd(H, H, std=0.3)).to(torch.bfloat16).float()})
         else:
             H, D, Dv = m["heads"], m["dim"], m["vdim"]
@@ -173,7 +174,7 @@ def random_tensors(cfg: LokizenConfig, seed: int = 0, rel_rows: int = 16) -> Dic
                       p + "mix.o": lin(W, H * Dv)})
         if L.get("mlp") is not None:
             E, ff = L["mlp"]["router"]["experts"], L["mlp"]["expert"]["ff"]
-            t[p + "norm2"] = 1 + rnd(W, std=0.1)
+            t[p + "norm2"] = one(W)
             t[p + "mlp.router"] = lin(E, W) * 2
             t[p + "mlp.correction"] = rnd(E, std=0.1)
             for e in range(E):
