@@ -69,11 +69,22 @@ JL_API int jl_attn_tile_rows(int32_t H, int32_t G, int32_t D, int32_t Dv);
  *   out_h(t) = o_t / sqrt(mean(o_t^2) + eps) * silu(gate_h(t))
  * proj [N, ld] holds q, k (H*D columns each), v and gate (H*Dv each) at the given columns.  state [slots, H, D, Dv] float: a request
  * with pos0 == 0 starts from zero (its slot's old content is ignored), otherwise from state[slot]; the final state is written
- * back.  seq [B, 4] int32 as above. */
+ * back.  seq [B, 4] int32 as above.
+ *
+ * `mode` JL_RET_SCAN is that.  Long portions are cut into chunks that run side by side in three launches: JL_RET_LOCAL_STATE (the
+ * records are chunks, `state` a scratch [chunks, H, D, Dv] indexed by the record's slot: each chunk's own contribution from a zero
+ * state, no output), jl_retention_join (turns the contributions into the state every chunk starts from and writes the requests'
+ * final states), JL_RET_FROM_SLOT (chunks again: outputs from the scratch's start states, nothing stored). */
+#define JL_RET_SCAN 0
+#define JL_RET_LOCAL_STATE 1
+#define JL_RET_FROM_SLOT 2
 JL_API int jl_retention(const void *proj, int dtype, int64_t ld, int32_t q_col, int32_t k_col, int32_t v_col, int32_t g_col,
                         const int32_t *seq, int32_t B, int32_t H, int32_t D, int32_t Dv, int32_t rot_dims, const float *cos_t,
                         const float *sin_t, int64_t table_len, const float *decay, float eps, float *state, void *out,
-                        void *stream);
+                        int32_t mode, void *stream);
+/* req [B, 4] int32 = {first chunk, chunks, pos0, slot}; chunk_len [chunks] int32; scratch [chunks, H, D, Dv] float as above. */
+JL_API int jl_retention_join(const int32_t *req, int32_t B, const int32_t *chunk_len, int32_t H, int32_t D, int32_t Dv,
+                             const float *decay, float *state, float *scratch, void *stream);
 
 /* Router of a mixture of experts: s = sigmoid(logits) (float [N, E]); the `top` experts with the largest s + correction are
  * chosen (ties: lowest index); ids [N, top] int32, weights [N, top] float = s * scale (not renormalised). */

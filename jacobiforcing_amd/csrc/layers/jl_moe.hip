@@ -1,5 +1,6 @@
 // jl_moe.hip — routed experts: the router's choice, the rows grouped by expert, and the two grouped products around relu^2.
 #include "jl_common.h"
+#include <stdlib.h>
 
 // ---- router: one thread per token ------------------------------------------------------------------------------------------------
 __global__ __launch_bounds__(256) void moe_route_kernel(const float *__restrict__ logits, const float *__restrict__ correction, int64_t N,
@@ -33,7 +34,7 @@ extern "C" int jl_moe_route(const float *logits, const float *correction, int64_
 }
 
 // ---- grouping: one workgroup counts, scans and places (a step holds at most a few 10^5 rows) ----------------------------------------
-constexpr int MOE_TM = 32;        // rows of a tile
+constexpr int MOE_TM = 64;        // rows of a tile
 constexpr int MOE_TN = 64;        // output columns of a tile
 constexpr int MOE_TK = 32;        // depth of one LDS stage
 constexpr int MOE_MAX_E = 4096;
@@ -60,13 +61,13 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int32_t *__restri
         for (; t < max_tiles; ++t) { tile_expert[t] = -1; tile_row0[t] = 0; }
     }
     __syncthreads();
-    // placement in row order within an expert, one thread per expert scanning the list (all reads hit L2): the order is fixed, so a
-    // run is reproducible
-    for (int e = threadIdx.x; e < E; e += 1024) {
-        int o = base[e];
-        if (cnt[e])
-            for (int64_t r = 0; r < rows; ++r)
-                if (ids[r] == e) perm[o++] = (int32_t)r;
+    // placement: a row's place within its expert is whatever the counter says when it arrives.  The order of an expert's rows
+    // changes nothing in the results (every row is computed by itself); only which tile a row lands in differs from run to run.
+    for (int e = threadIdx.x; e < E; e += 1024) cnt[e] = 0;
+    __syncthreads();
+    for (int64_t r = threadIdx.x; r < rows; r += 1024) {
+        const int e = ids[r];
+        perm[base[e] + atomicAdd(&cnt[e], 1)] = (int32_t)r;
     }
 }
 
@@ -82,7 +83,7 @@ extern "C" int jl_moe_group(const int32_t *ids, int64_t N, int32_t top, int32_t 
     return jl_check_launch("moe_group_kernel");
 }
 
-// ---- grouped product: a 32 x 64 tile of one expert's rows per workgroup, products in float from float / bf16 operands -------------------
+// ---- grouped product, any dtype and size: a 64 x 64 tile of one expert's rows per workgroup, float FMAs ------------------------------------
 template <typename T>
 __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, const T *__restrict__ Wt, int mode, int K, int n_out, int top,
                                                         const int32_t *__restrict__ perm, const int32_t *__restrict__ offsets,
@@ -99,7 +100,7 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, 
     const int tid = threadIdx.x, ty = tid >> 4, tx = tid & 15;
     if (tid < MOE_TM) rin[tid] = tid < nr ? (mode == 0 ? perm[r0 + tid] / top : r0 + tid) : -1;
     const T *We = Wt + (int64_t)e * n_out * K;
-    float acc[2][4] = {{0.f, 0.f, 0.f, 0.f}, {0.f, 0.f, 0.f, 0.f}};
+    float acc[4][4] = {};
     for (int k0 = 0; k0 < K; k0 += MOE_TK) {
         __syncthreads();
         for (int i = tid; i < MOE_TM * MOE_TK; i += 256) {
@@ -113,18 +114,20 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, 
         __syncthreads();
 #pragma unroll 8
         for (int kk = 0; kk < MOE_TK; ++kk) {
-            const float a0 = Xs[ty * 2][kk], a1 = Xs[ty * 2 + 1][kk];
+            float av[4];
+#pragma unroll
+            for (int a = 0; a < 4; ++a) av[a] = Xs[ty + 16 * a][kk];
 #pragma unroll
             for (int c = 0; c < 4; ++c) {
                 const float w = Ws[tx + 16 * c][kk];
-                acc[0][c] += a0 * w;
-                acc[1][c] += a1 * w;
+#pragma unroll
+                for (int a = 0; a < 4; ++a) acc[a][c] += av[a] * w;
             }
         }
     }
 #pragma unroll
-    for (int a = 0; a < 2; ++a) {
-        const int m = ty * 2 + a;
+    for (int a = 0; a < 4; ++a) {
+        const int m = ty + 16 * a;
         if (m >= nr) continue;
         const int r = r0 + m;
 #pragma unroll
@@ -142,6 +145,87 @@ __global__ __launch_bounds__(256) void moe_gemm_kernel(const T *__restrict__ X, 
     }
 }
 
+// ---- grouped product on the matrix cores (bfloat16, K a multiple of 8) -----------------------------------------------------------------
+// A 64 x 128 tile per workgroup, four wavefronts side by side over the columns: each holds two 32 x 32 accumulators (rows 0-31 and
+// 32-63) and feeds v_mfma_f32_32x32x8_bf16 from LDS stages of depth 32.  Operand layout of that instruction: lane l supplies row
+// (A) or column (B) l % 32 with the four consecutive depths 4 * (l / 32) ..; accumulator i of lane l is row 8 * (i / 4) + 4 * (l / 32)
+// + i % 4, column l % 32.
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short bf16x4_t;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float f32x16_t;
+constexpr int MM_TN = 128, MM_TK = 32, MM_LD = 36;     // LDS row stride in bf16 (72 bytes: rows 16 apart share a bank, no worse)
+
+__global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__restrict__ X, const bf16_t *__restrict__ Wt, int mode, int K, int n_out,
+                                                             int top, const int32_t *__restrict__ perm, const int32_t *__restrict__ offsets,
+                                                             const int32_t *__restrict__ tile_expert, const int32_t *__restrict__ tile_row0,
+                                                             const float *__restrict__ weights, void *__restrict__ out) {
+    __shared__ __attribute__((aligned(16))) bf16_t As[MOE_TM * MM_LD];
+    __shared__ __attribute__((aligned(16))) bf16_t Bs[MM_TN * MM_LD];
+    __shared__ int rin[MOE_TM];
+    const int e = tile_expert[blockIdx.x];
+    if (e < 0) return;
+    const int r0 = tile_row0[blockIdx.x];
+    const int nr = offsets[e + 1] - r0 < MOE_TM ? offsets[e + 1] - r0 : MOE_TM;
+    const int n0 = blockIdx.y * MM_TN;
+    const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63;
+    if (tid < MOE_TM) rin[tid] = tid < nr ? (mode == 0 ? perm[r0 + tid] / top : r0 + tid) : -1;
+    __syncthreads();
+    const bf16_t *We = Wt + (int64_t)e * n_out * K;
+    // loaders: 8 bf16 (16 bytes) per thread and row segment; A 64 x 32 = 256 segments, B 128 x 32 = 512 segments
+    const int a_row = tid >> 2, a_seg = (tid & 3) * 8;
+    const int64_t a_src = rin[a_row] >= 0 ? (int64_t)rin[a_row] * K : -1;
+    f32x16_t acc0 = {0}, acc1 = {0};
+    for (int k0 = 0; k0 < K; k0 += MM_TK) {
+        uint4 av = make_uint4(0, 0, 0, 0), bv[2];
+        if (a_src >= 0 && k0 + a_seg < K) av = *(const uint4 *)(X + a_src + k0 + a_seg);
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            const int n = (tid >> 2) + 64 * i;
+            bv[i] = make_uint4(0, 0, 0, 0);
+            if (n0 + n < n_out && k0 + a_seg < K) bv[i] = *(const uint4 *)(We + (int64_t)(n0 + n) * K + k0 + a_seg);
+        }
+        __syncthreads();                                   // the previous stage's readers are done
+        {
+            uint2 *d = (uint2 *)(As + a_row * MM_LD + a_seg);       // rows are 72 bytes apart: 8-byte stores stay aligned
+            d[0] = make_uint2(av.x, av.y);
+            d[1] = make_uint2(av.z, av.w);
+        }
+#pragma unroll
+        for (int i = 0; i < 2; ++i) {
+            uint2 *d = (uint2 *)(Bs + ((tid >> 2) + 64 * i) * MM_LD + a_seg);
+            d[0] = make_uint2(bv[i].x, bv[i].y);
+            d[1] = make_uint2(bv[i].z, bv[i].w);
+        }
+        __syncthreads();
+#pragma unroll
+        for (int kk = 0; kk < MM_TK; kk += 8) {
+            const int ko = kk + 4 * (lane >> 5);
+            const bf16x4_t b = *(const bf16x4_t *)(Bs + (wave * 32 + (lane & 31)) * MM_LD + ko);
+            const bf16x4_t a0 = *(const bf16x4_t *)(As + (lane & 31) * MM_LD + ko);
+            const bf16x4_t a1 = *(const bf16x4_t *)(As + (32 + (lane & 31)) * MM_LD + ko);
+            acc0 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a0, b, acc0, 0, 0, 0);
+            acc1 = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(a1, b, acc1, 0, 0, 0);
+        }
+    }
+    const int n = n0 + wave * 32 + (lane & 31);
+    if (n >= n_out) return;
+#pragma unroll
+    for (int half = 0; half < 2; ++half)
+#pragma unroll
+        for (int i = 0; i < 16; ++i) {
+            const int m = 32 * half + 8 * (i >> 2) + 4 * (lane >> 5) + (i & 3);
+            if (m >= nr) continue;
+            const float c = half ? acc1[i] : acc0[i];
+            const int r = r0 + m;
+            if (mode == 0) {
+                const float v = fmaxf(c, 0.f);
+                st_f((bf16_t *)out + (int64_t)r * n_out + n, v * v);
+            } else {
+                const int p = perm[r];
+                ((float *)out)[(int64_t)p * n_out + n] = c * weights[p];
+            }
+        }
+}
+
 extern "C" int jl_moe_gemm(const void *X, const void *Wt, int dtype, int32_t mode, int32_t K, int32_t n_out, int32_t top,
                            const int32_t *perm, const int32_t *offsets, const int32_t *tile_expert, const int32_t *tile_row0,
                            int32_t max_tiles, const float *weights, void *out, void *stream) {
@@ -149,6 +233,13 @@ extern "C" int jl_moe_gemm(const void *X, const void *Wt, int dtype, int32_t mod
     if (!X || !Wt || !perm || !offsets || !tile_expert || !tile_row0 || !out || (mode == 1 && !weights))
         return jl_fail(JL_E_INVALID, "jl_moe_gemm: null pointer");
     if (K <= 0 || n_out <= 0 || top <= 0 || (mode != 0 && mode != 1)) return jl_fail(JL_E_INVALID, "jl_moe_gemm: bad sizes or mode");
+    static const bool no_mfma = getenv("JL_MOE_NO_MFMA") != nullptr;      // A/B switch for measurements
+    if (!no_mfma && dtype == JL_BF16 && K % 8 == 0 && ((uintptr_t)X % 16) == 0 && ((uintptr_t)Wt % 16) == 0) {
+        const dim3 mgrid((unsigned)max_tiles, (unsigned)((n_out + MM_TN - 1) / MM_TN));
+        moe_gemm_mfma_kernel<<<mgrid, 256, 0, (hipStream_t)stream>>>((const bf16_t *)X, (const bf16_t *)Wt, mode, K, n_out, top, perm, offsets,
+                                                                    tile_expert, tile_row0, weights, out);
+        return jl_check_launch("moe_gemm_mfma_kernel");
+    }
     const dim3 grid((unsigned)max_tiles, (unsigned)((n_out + MOE_TN - 1) / MOE_TN));
     JL_DISPATCH(dtype, moe_gemm_kernel<T><<<grid, 256, 0, (hipStream_t)stream>>>((const T *)X, (const T *)Wt, mode, K, n_out, top, perm, offsets,
                                                                                  tile_expert, tile_row0, weights, out));

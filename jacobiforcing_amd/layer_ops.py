@@ -15,6 +15,9 @@ import torch
 from . import _native as N
 
 
+RETENTION_CHUNK = 64          # tokens per chunk when a long portion's recurrence is cut into chunks that run side by side
+
+
 def _ptr(t: Optional[torch.Tensor]):
     return None if t is None else C.c_void_p(t.data_ptr())
 
@@ -80,6 +83,27 @@ class RaggedBatch:
                    seq=torch.from_numpy(seq).to(dev), kv_slot=torch.from_numpy(kv).to(dev), tables=torch.from_numpy(bt).to(dev),
                    page_size=int(page_size), max_pos=max(int(s) + int(c) for s, c in zip(starts, counts)), max_page=int(bt.max()),
                    max_slot=int(max(slots)), _tiles={})
+
+    def chunks(self, size: int):
+        """A portion of at least two chunks is cut into chunks of ``size`` tokens that the recurrent layers run side by side.
+        None when no request of the step is that long.  Else (chunk records [chunks, 4] int32 {row0, count, pos0, chunk index},
+        chunk lengths [chunks] int32, request records [B, 4] int32 {first chunk, chunks, pos0, slot})."""
+        key = ("chunks", size)
+        if key not in self._tiles:
+            plan = None
+            if max(self.counts) >= 2 * size:
+                seq = self.seq.cpu().numpy()
+                rec, req = [], []
+                for b, (c, s) in enumerate(zip(self.counts, self.starts)):
+                    req.append((len(rec), -(-c // size), s, int(seq[b, 3])))
+                    for o in range(0, c, size):
+                        rec.append((int(seq[b, 0]) + o, min(size, c - o), s + o, len(rec)))
+                dev = self.seq.device
+                rec = np.asarray(rec, dtype=np.int32).reshape(-1, 4)
+                plan = (torch.from_numpy(rec).to(dev), torch.from_numpy(np.ascontiguousarray(rec[:, 1])).to(dev),
+                        torch.from_numpy(np.asarray(req, dtype=np.int32).reshape(-1, 4)).to(dev))
+            self._tiles[key] = plan
+        return self._tiles[key]
 
     def tiles(self, tq: int) -> torch.Tensor:
         """[n_tiles, 4] int32 {b, first query position, count, first row}: each request's rows cut into runs of at most ``tq``."""
@@ -198,9 +222,21 @@ def retention(proj: torch.Tensor, cols: Tuple[int, int, int, int], batch: Ragged
         tl = cos.shape[0]
         _need(batch.max_pos <= tl, "retention: the angle tables are shorter than the batch's positions")
     out = torch.empty((n, H * Dv), dtype=proj.dtype, device=proj.device)
-    N.check_layers(N.layers().jl_retention(_ptr(proj), _code(proj.dtype), ld, cols[0], cols[1], cols[2], cols[3], _ptr(batch.seq), batch.B, H, D, Dv,
-                                          rot_dims, _ptr(cos), _ptr(sin), tl, _ptr(decay), float(eps), _ptr(state), _ptr(out),
-                                          _stream(proj.device)), "jl_retention")
+    L, st = N.layers(), _stream(proj.device)
+
+    def scan(records, count, where, mode, what):
+        N.check_layers(L.jl_retention(_ptr(proj), _code(proj.dtype), ld, cols[0], cols[1], cols[2], cols[3], _ptr(records), count, H, D, Dv,
+                                      rot_dims, _ptr(cos), _ptr(sin), tl, _ptr(decay), float(eps), _ptr(where), _ptr(out), mode, st), what)
+
+    plan = batch.chunks(RETENTION_CHUNK)
+    if plan is None:                                    # decoded tokens and short portions: one scan per request
+        scan(batch.seq, batch.B, state, 0, "jl_retention")
+        return out
+    chunk_rec, chunk_len, req = plan
+    scratch = torch.empty((chunk_rec.shape[0], H, D, Dv), dtype=torch.float32, device=proj.device)
+    scan(chunk_rec, chunk_rec.shape[0], scratch, 1, "jl_retention(local state)")
+    N.check_layers(L.jl_retention_join(_ptr(req), batch.B, _ptr(chunk_len), H, D, Dv, _ptr(decay), _ptr(state), _ptr(scratch), st), "jl_retention_join")
+    scan(chunk_rec, chunk_rec.shape[0], scratch, 2, "jl_retention(outputs)")
     return out
 
 
