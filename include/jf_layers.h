@@ -60,8 +60,8 @@ typedef struct {
     float scale;
 } jl_attn_args;
 JL_API int jl_attn_window(const jl_attn_args *a, void *stream);
-/* largest TQ (query rows per tile) the kernel takes for these sizes */
-JL_API int jl_attn_tile_rows(int32_t H, int32_t G, int32_t D, int32_t Dv);
+/* TQ (query rows per tile) the kernel wants for this dtype and these sizes; 0 when they do not fit */
+JL_API int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv);
 
 /* Retention (linear attention with a fixed decay per head, no denominator) over the ragged batch, state carried in float:
  *   q, k rotated (rotate-half pairs on the first rot_dims dimensions, angles from the cos / sin tables [positions, rot_dims/2]),

@@ -249,7 +249,7 @@ _LAYER_SIGNATURES = {
     "jl_add_rmsnorm": (C.c_int, [_vp, _vp, C.c_int, _i32, _vp, _vp, _f32, _vp, C.c_int, _i64, _i32, _vp]),
     "jl_qk_norm_append": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),
     "jl_attn_window": (C.c_int, [C.POINTER(AttnArgs), _vp]),
-    "jl_attn_tile_rows": (C.c_int, [_i32, _i32, _i32, _i32]),
+    "jl_attn_tile_rows": (C.c_int, [C.c_int, _i32, _i32, _i32, _i32]),
     "jl_retention": (C.c_int, [_vp, C.c_int, _i64, _i32, _i32, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _f32,
                                _vp, _vp, _i32, _vp]),
     "jl_retention_join": (C.c_int, [_vp, _i32, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp]),

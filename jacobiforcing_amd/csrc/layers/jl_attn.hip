@@ -1,6 +1,7 @@
 // jl_attn.hip — query / key norm + paged append, and attention with a sliding window that keeps the first tokens, a bucketed
 // distance bias and mixed heads, for prompt portions and single decoded tokens alike (one ragged launch).
 #include "jl_common.h"
+#include <stdlib.h>
 
 // ---- whole-projection q / k norm + append: one workgroup per token ------------------------------------------------------------
 template <typename T>
@@ -68,7 +69,11 @@ static bool att_shape(int H, int G, int D, int Dv, int tq_want, AttShape *o) {
     return false;
 }
 
-extern "C" int jl_attn_tile_rows(int32_t H, int32_t G, int32_t D, int32_t Dv) {
+static bool am_fits(int dtype, int H, int G, int D, int Dv);
+
+extern "C" int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv) {
+    if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0) return 0;
+    if (am_fits(dtype, H, G, D, Dv)) return 32;
     AttShape s;
     return att_shape(H, G, D, Dv, 0, &s) ? s.TQ : 0;
 }
@@ -201,6 +206,240 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
     }
 }
 
+// ---- the same attention on the matrix cores (bfloat16; H <= 16, D a multiple of 8 up to 256, Dv up to 128) -----------
+// A tile of 32 query rows of one request, all heads; wavefront w owns heads w * HPW .. (HPW = 1 or 2).  Keys go through LDS 32 at a
+// time.  v_mfma_f32_32x32x8_bf16: lane l supplies row (A) or column (B) l % 32 with depths 4 * (l / 32) .. + 3; accumulator r of lane
+// l is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32.
+//   sweep 1: S = Q K^T per own head; every lane keeps a running maximum and sum for its 16 rows over its column; merged over the
+//            lanes at the end -> maximum and 1 / sum per (head, row) in LDS.
+//   sweep 2: S again -> p = exp(s - max) / sum in float -> LDS, all heads; after a barrier every wavefront mixes the heads'
+//            weights for its own heads directly in the A-operand layout (w = sum_g talk[h, g] p_g, float, rounded once to
+//            bfloat16) and multiplies by the value tile.
+typedef __attribute__((__vector_size__(4 * sizeof(short)))) short am_bf16x4;
+typedef __attribute__((__vector_size__(16 * sizeof(float)))) float am_f32x16;
+constexpr int AM_T = 32;
+
+__device__ __forceinline__ short am_bf16(float v) {
+    uint32_t u = __float_as_uint(v);
+    u += 0x7FFFu + ((u >> 16) & 1u);
+    return (short)(u >> 16);
+}
+
+static size_t am_lds_bytes(int H, int G, int D, int Dv) {
+    return (size_t)G * AM_T * (D + 4) * 2 + (size_t)AM_T * G * Dv * 2 + ((size_t)H * AM_T * 33 + 2 * (size_t)H * AM_T + (size_t)H * H) * 4;
+}
+
+template <int HPW, int NDV>
+__global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a) {
+    extern __shared__ __attribute__((aligned(16))) char smem[];
+    const int H = a.H, G = a.G, D = a.D, Dv = a.Dv, rep = H / G, KLD = D + 4;
+    const int tid = threadIdx.x, nthr = blockDim.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, hi = lane >> 5;
+    const int *tile = a.tiles + 4 * (int64_t)blockIdx.x;
+    const int b = tile[0], i0 = tile[1], cnt = tile[2], row0 = tile[3];
+    if (b < 0 || cnt <= 0) return;
+    bf16_t *Ks = (bf16_t *)smem;                                   // [G][32][D + 4]
+    bf16_t *Vs = Ks + G * AM_T * KLD;                              // [32][G * Dv]
+    float *Ps = (float *)(Vs + AM_T * G * Dv);                     // [H][32][33]
+    float *mS = Ps + H * AM_T * 33;                                // [H][32] row maximum
+    float *lS = mS + H * AM_T;                                     // [H][32] 1 / row sum
+    float *talk = lS + H * AM_T;                                   // [H][H]
+    const int window = a.window > 0 ? a.window : 0x3fffffff;
+    const int i_max = i0 + cnt - 1;
+    const int lo = i0 - window + 1 > 0 ? i0 - window + 1 : 0;
+    const int kf_end = a.keep_first < lo ? a.keep_first : lo;
+    const int n_keys = kf_end + (i_max + 1 - lo);
+    const int *bt = a.block_tables + (int64_t)b * a.bt_stride;
+    const bf16_t *q = (const bf16_t *)a.q, *kc = (const bf16_t *)a.k_cache, *vc = (const bf16_t *)a.v_cache;
+    if (a.talk) for (int e = tid; e < H * H; e += nthr) talk[e] = a.talk[e];
+
+    float m_run[HPW][16], l_run[HPW][16];
+    am_f32x16 acc[HPW][NDV];
+#pragma unroll
+    for (int x = 0; x < HPW; ++x) {
+#pragma unroll
+        for (int r = 0; r < 16; ++r) { m_run[x][r] = -INFINITY; l_run[x][r] = 0.f; }
+#pragma unroll
+        for (int t = 0; t < NDV; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[x][t][r] = 0.f;
+    }
+
+    for (int sweep = 0; sweep < 2; ++sweep) {
+        for (int u0 = 0; u0 < n_keys; u0 += AM_T) {
+            const int nk = n_keys - u0 < AM_T ? n_keys - u0 : AM_T;
+            __syncthreads();                                        // the previous tile's readers are done
+            const int kq = G * D / 4;                               // 8-byte units per key
+            for (int e = tid; e < AM_T * kq; e += nthr) {
+                const int jj = e / kq, r = e - jj * kq, c = r / (D / 4), d4 = r - c * (D / 4);
+                uint2 v = make_uint2(0, 0);
+                if (jj < nk) {
+                    const int u = u0 + jj, j = u < kf_end ? u : lo + (u - kf_end);
+                    const int64_t tok = (int64_t)bt[j / a.page_size] * a.page_size + j % a.page_size;
+                    v = *(const uint2 *)(kc + tok * (G * D) + 4 * r);
+                }
+                *(uint2 *)(Ks + (c * AM_T + jj) * KLD + 4 * d4) = v;
+            }
+            if (sweep == 1) {
+                const int vq = G * Dv / 4;
+                for (int e = tid; e < AM_T * vq; e += nthr) {
+                    const int jj = e / vq, r = e - jj * vq;
+                    uint2 v = make_uint2(0, 0);
+                    if (jj < nk) {
+                        const int u = u0 + jj, j = u < kf_end ? u : lo + (u - kf_end);
+                        const int64_t tok = (int64_t)bt[j / a.page_size] * a.page_size + j % a.page_size;
+                        v = *(const uint2 *)(vc + tok * (G * Dv) + 4 * r);
+                    }
+                    *(uint2 *)(Vs + jj * (G * Dv) + 4 * r) = v;
+                }
+            }
+            __syncthreads();
+            // this lane's key (column l32 of the tile)
+            const int u = u0 + l32, j = u < kf_end ? u : lo + (u - kf_end);
+#pragma unroll
+            for (int x = 0; x < HPW; ++x) {
+                const int g = wave * HPW + x;
+                if (g >= H) continue;
+                const int c = g / rep;
+                am_f32x16 sc;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) sc[r] = 0.f;
+                const bf16_t *qp = q + (int64_t)(row0 + l32) * (H * D) + g * D + 4 * hi;
+                const bf16_t *kp = Ks + (c * AM_T + l32) * KLD + 4 * hi;
+                for (int kk = 0; kk < D; kk += 8) {
+                    am_bf16x4 qa = {0, 0, 0, 0};
+                    if (l32 < cnt) qa = *(const am_bf16x4 *)(qp + kk);
+                    const am_bf16x4 kb = *(const am_bf16x4 *)(kp + kk);
+                    sc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(qa, kb, sc, 0, 0, 0);
+                }
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int ii = 8 * (r >> 2) + 4 * hi + (r & 3), i = i0 + ii;
+                    const bool ok = ii < cnt && l32 < nk && j <= i && (i - j < window || j < a.keep_first);
+                    float s = -INFINITY;
+                    if (ok) {
+                        s = sc[r] * a.scale;
+                        if (a.rel) {
+                            const int n = i - j < a.lut_len ? i - j : a.lut_len - 1;
+                            s += a.rel[a.lut[n] * H + g];
+                        }
+                    }
+                    if (sweep == 0) {
+                        const float t = fmaxf(m_run[x][r], s);
+                        if (t > -INFINITY) {
+                            l_run[x][r] = l_run[x][r] * __expf(m_run[x][r] - t) + __expf(s - t);
+                            m_run[x][r] = t;
+                        }
+                    } else {
+                        Ps[(g * AM_T + ii) * 33 + l32] = ok ? __expf(s - mS[g * AM_T + ii]) * lS[g * AM_T + ii] : 0.f;
+                    }
+                }
+            }
+            if (sweep == 0) continue;
+            __syncthreads();
+            // mixed weights of the own heads in the A layout (row l32, keys 8 s + 4 hi ..), times the values
+#pragma unroll
+            for (int sK = 0; sK < AM_T / 8; ++sK) {
+                const int j0 = 8 * sK + 4 * hi;
+                float w[HPW][4];
+#pragma unroll
+                for (int x = 0; x < HPW; ++x)
+#pragma unroll
+                    for (int qd = 0; qd < 4; ++qd) w[x][qd] = 0.f;
+                if (a.talk) {
+                    for (int g = 0; g < H; ++g) {
+                        const float *pp = Ps + (g * AM_T + l32) * 33 + j0;
+                        const float p0 = pp[0], p1 = pp[1], p2 = pp[2], p3 = pp[3];
+#pragma unroll
+                        for (int x = 0; x < HPW; ++x) {
+                            const int h = wave * HPW + x;
+                            const float tw = h < H ? talk[h * H + g] : 0.f;
+                            w[x][0] += tw * p0; w[x][1] += tw * p1; w[x][2] += tw * p2; w[x][3] += tw * p3;
+                        }
+                    }
+                } else {
+#pragma unroll
+                    for (int x = 0; x < HPW; ++x) {
+                        const int h = wave * HPW + x;
+                        if (h < H)
+#pragma unroll
+                            for (int qd = 0; qd < 4; ++qd) w[x][qd] = Ps[(h * AM_T + l32) * 33 + j0 + qd];
+                    }
+                }
+#pragma unroll
+                for (int x = 0; x < HPW; ++x) {
+                    const int h = wave * HPW + x;
+                    if (h >= H) continue;
+                    const int c = h / rep;
+                    const am_bf16x4 wa = {am_bf16(w[x][0]), am_bf16(w[x][1]), am_bf16(w[x][2]), am_bf16(w[x][3])};
+#pragma unroll
+                    for (int t = 0; t < NDV; ++t) {
+                        if (32 * t >= Dv) continue;
+                        const bf16_t *vp = Vs + j0 * (G * Dv) + c * Dv + 32 * t + l32;
+                        const am_bf16x4 vb = {(short)vp[0], (short)vp[G * Dv], (short)vp[2 * G * Dv], (short)vp[3 * G * Dv]};
+                        acc[x][t] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(wa, vb, acc[x][t], 0, 0, 0);
+                    }
+                }
+            }
+        }
+        if (sweep == 0) {
+            // merge the lanes' running statistics: rows are shared by the 32 lanes of a half wavefront
+#pragma unroll
+            for (int x = 0; x < HPW; ++x) {
+                const int g = wave * HPW + x;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    float M = m_run[x][r];
+#pragma unroll
+                    for (int off = 16; off > 0; off >>= 1) M = fmaxf(M, __shfl_xor(M, off, 64));
+                    float L = M > -INFINITY ? l_run[x][r] * __expf(m_run[x][r] - M) : 0.f;
+#pragma unroll
+                    for (int off = 16; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
+                    const int ii = 8 * (r >> 2) + 4 * hi + (r & 3);
+                    if (l32 == 0 && g < H) { mS[g * AM_T + ii] = M; lS[g * AM_T + ii] = L > 0.f ? 1.0f / L : 0.f; }
+                }
+            }
+        }
+    }
+    bf16_t *out = (bf16_t *)a.out;
+    const bf16_t *gate = (const bf16_t *)a.gate;
+#pragma unroll
+    for (int x = 0; x < HPW; ++x) {
+        const int h = wave * HPW + x;
+        if (h >= H) continue;
+#pragma unroll
+        for (int t = 0; t < NDV; ++t) {
+            if (32 * t + l32 >= Dv) continue;                       // a last column tile may be partly beyond Dv: computed, never stored
+#pragma unroll
+            for (int r = 0; r < 16; ++r) {
+                const int ii = 8 * (r >> 2) + 4 * hi + (r & 3);
+                if (ii >= cnt) continue;
+                const int col = h * Dv + 32 * t + l32;
+                float v = acc[x][t][r];
+                if (gate) v *= 1.0f / (1.0f + __expf(-ld_f(gate + (int64_t)(row0 + ii) * a.gate_ld + col)));
+                st_f(out + (int64_t)(row0 + ii) * (H * Dv) + col, v);
+            }
+        }
+    }
+}
+
+static bool am_fits(int dtype, int H, int G, int D, int Dv) {
+    static const bool off = getenv("JL_ATTN_NO_MFMA") != nullptr;          // A/B switch for measurements
+    return !off && dtype == JL_BF16 && H <= 16 && D % 8 == 0 && D <= 256 && Dv <= 128 && (G * Dv) % 4 == 0 &&
+           am_lds_bytes(H, G, D, Dv) <= (size_t)ATT_LDS_BUDGET + 8 * 1024;
+}
+
+template <int HPW, int NDV> static int am_launch(const jl_attn_args &a, hipStream_t st) {
+    auto kern = attn_mfma_kernel<HPW, NDV>;
+    const size_t lds = am_lds_bytes(a.H, a.G, a.D, a.Dv);
+    if (lds > 64 * 1024) {
+        hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);
+        if (e != hipSuccess) return jl_fail(JL_E_LAUNCH, "jl_attn_window: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
+    }
+    const int waves = (a.H + HPW - 1) / HPW;
+    kern<<<dim3((unsigned)a.n_tiles), 64 * waves, lds, st>>>(a);
+    return jl_check_launch("attn_mfma_kernel");
+}
+
 template <typename T, int ACC> static int att_launch(const jl_attn_args &a, const AttShape &s, hipStream_t st) {
     auto kern = attn_window_kernel<T, ACC>;
     if (s.lds > 64 * 1024) {
@@ -219,10 +458,17 @@ extern "C" int jl_attn_window(const jl_attn_args *ap, void *stream) {
     if (a.H <= 0 || a.G <= 0 || a.H % a.G || a.D <= 0 || a.Dv <= 0 || a.page_size <= 0 || a.TQ <= 0)
         return jl_fail(JL_E_INVALID, "jl_attn_window: bad head counts or sizes");
     if ((a.rel != nullptr) != (a.lut != nullptr) || (a.lut && a.lut_len <= 0)) return jl_fail(JL_E_INVALID, "jl_attn_window: rel and lut come together");
+    hipStream_t st = (hipStream_t)stream;
+    if (a.TQ == AM_T && am_fits(a.dtype, a.H, a.G, a.D, a.Dv)) {
+        const int ndv = (a.Dv + 31) / 32;
+#define AM_CASE(HP, ND) if ((a.H > 8 ? 2 : 1) == HP && ndv == ND) return am_launch<HP, ND>(a, st)
+        AM_CASE(1, 1); AM_CASE(1, 2); AM_CASE(1, 3); AM_CASE(1, 4);
+        AM_CASE(2, 1); AM_CASE(2, 2); AM_CASE(2, 3); AM_CASE(2, 4);
+#undef AM_CASE
+    }
     AttShape s;
     if (!att_shape(a.H, a.G, a.D, a.Dv, a.TQ, &s) || s.TQ != a.TQ)
         return jl_fail(JL_E_INVALID, "jl_attn_window: TQ %d does not fit these sizes (ask jl_attn_tile_rows)", a.TQ);
-    hipStream_t st = (hipStream_t)stream;
 #define ATT_CASE(N) case N: JL_DISPATCH(a.dtype, return (att_launch<T, N>(a, s, st))); break
     switch (s.ACC) {
         ATT_CASE(16);

@@ -167,8 +167,8 @@ def qk_norm_append(proj: torch.Tensor, cols: Tuple[int, int, int], H: int, G: in
     return q
 
 
-def attn_tile_rows(H: int, G: int, D: int, Dv: int) -> int:
-    tq = int(N.layers().jl_attn_tile_rows(H, G, D, Dv))
+def attn_tile_rows(dtype: torch.dtype, H: int, G: int, D: int, Dv: int) -> int:
+    tq = int(N.layers().jl_attn_tile_rows(_code(dtype), H, G, D, Dv))
     if tq <= 0:
         raise ValueError(f"attention sizes heads={H} kv_heads={G} dim={D} vdim={Dv} exceed the kernel's tile")
     return tq
@@ -192,7 +192,7 @@ def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Te
             _need(t.dtype == torch.float32 and t.is_contiguous() and (shape is None or tuple(t.shape) == shape), "attn_window: float tables")
     if rel is not None:
         _need(lut is not None and lut.dtype == torch.int32 and rel.shape[1] == H, "attn_window: rel [rows, H] with its lut")
-    tq = attn_tile_rows(H, G, D, Dv)
+    tq = attn_tile_rows(dt, H, G, D, Dv)
     tiles = batch.tiles(tq)
     out = torch.empty((n, H * Dv), dtype=dt, device=q.device)
     a = N.AttnArgs(q=q.data_ptr(), gate=gate.data_ptr() if gate is not None else None, gate_ld=gate.stride(0) if gate is not None else 0,

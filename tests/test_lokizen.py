@@ -400,6 +400,31 @@ def test_long_portions_run_in_chunks(dtype, tol):
 
 
 @gpu
+@pytest.mark.parametrize("H,G,D,Dv", [(12, 4, 64, 128), (8, 2, 128, 64), (3, 1, 24, 40), (16, 16, 32, 32), (5, 5, 8, 100)])
+def test_attention_on_the_matrix_cores(H, G, D, Dv):
+    """bfloat16 attention alone (the MFMA kernel: one or two heads per wavefront, value widths that are no multiple of its
+    32-column tiles) on bfloat16-rounded inputs: two portions that cut a window, then single tokens, pages out of order."""
+    import torch.nn.functional as F
+    cfg = make_cfg([dict(attn(heads=H, kv=G, dim=D, vdim=Dv, size=37, keep=5, bias_max=90, scale=D ** -0.5), mlp=None)], width=64, vocab=50)
+    rig = Rig(cfg, seed=H, dtype=torch.bfloat16, pages=32)
+    T = 110
+    g = torch.Generator().manual_seed(H + D)
+    h = torch.randn(T, 64, generator=g).bfloat16()
+    P = {k: v.double() for k, v in O.layer_tensors(rig.tensors, 0).items()}
+    want = O.attention_mixer(h.double(), P, cfg["layers"][0]["mixer"], rig.cfg.norm_eps)
+    pages = list(range(31, 31 - 14, -1))
+    rig.poison()
+    got, at = [], 0
+    for n in (70, 37, 1, 1, 1):
+        b = rig.LO.RaggedBatch.build([n], [at], [0], [pages], 8, "cuda")
+        got.append(F.linear(rig.model._attention(0, 0, h[at:at + n].cuda(), b, rig.cache), rig.model.w.layers[0]["w_o"]).float().cpu())
+        at += n
+    got = torch.cat(got)
+    assert rel_err(got, want) < 2e-2
+    assert max(rel_err(got[i], want[i]) for i in range(T)) < 6e-2
+
+
+@gpu
 def test_grouped_expert_products_on_the_matrix_cores():
     """bfloat16 with a depth that is a multiple of 8 takes the MFMA kernel: many rows per expert, experts without rows, row counts
     that are no multiple of the tile, output widths that are no multiple of 128."""
