@@ -58,7 +58,10 @@ typedef struct {
     const int32_t *block_tables; const int32_t *tiles; const float *rel; const int32_t *lut; const float *talk;
     int32_t bt_stride, n_tiles, lut_len, page_size, H, G, D, Dv, window, keep_first, TQ, dtype;
     float scale;
+    int32_t splits, n_rows;       /* splits > 1 (TQ 32 only): each tile's keys are shared out over `splits` workgroups — statistics, */
+    float *scratch;               /* outputs, join: three launches; scratch of jl_attn_scratch_floats() floats, n_rows = N          */
 } jl_attn_args;
+JL_API int64_t jl_attn_scratch_floats(int32_t n_tiles, int32_t n_rows, int32_t H, int32_t Dv, int32_t splits);
 JL_API int jl_attn_window(const jl_attn_args *a, void *stream);
 /* TQ (query rows per tile) the kernel wants for this dtype and these sizes; 0 when they do not fit */
 JL_API int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv);

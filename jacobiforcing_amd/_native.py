@@ -239,7 +239,8 @@ class AttnArgs(C.Structure):
     _fields_ = [("q", _vp), ("gate", _vp), ("gate_ld", _i64), ("k_cache", _vp), ("v_cache", _vp), ("out", _vp),
                 ("block_tables", _vp), ("tiles", _vp), ("rel", _vp), ("lut", _vp), ("talk", _vp),
                 ("bt_stride", _i32), ("n_tiles", _i32), ("lut_len", _i32), ("page_size", _i32), ("H", _i32), ("G", _i32), ("D", _i32),
-                ("Dv", _i32), ("window", _i32), ("keep_first", _i32), ("TQ", _i32), ("dtype", _i32), ("scale", _f32)]
+                ("Dv", _i32), ("window", _i32), ("keep_first", _i32), ("TQ", _i32), ("dtype", _i32), ("scale", _f32),
+                ("splits", _i32), ("n_rows", _i32), ("scratch", _vp)]
 
 
 _LAYER_SIGNATURES = {
@@ -249,6 +250,7 @@ _LAYER_SIGNATURES = {
     "jl_add_rmsnorm": (C.c_int, [_vp, _vp, C.c_int, _i32, _vp, _vp, _f32, _vp, C.c_int, _i64, _i32, _vp]),
     "jl_qk_norm_append": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),
     "jl_attn_window": (C.c_int, [C.POINTER(AttnArgs), _vp]),
+    "jl_attn_scratch_floats": (_i64, [_i32, _i32, _i32, _i32, _i32]),
     "jl_attn_tile_rows": (C.c_int, [C.c_int, _i32, _i32, _i32, _i32]),
     "jl_retention": (C.c_int, [_vp, C.c_int, _i64, _i32, _i32, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _f32,
                                _vp, _vp, _i32, _vp]),

@@ -71,6 +71,10 @@ static bool att_shape(int H, int G, int D, int Dv, int tq_want, AttShape *o) {
 
 static bool am_fits(int dtype, int H, int G, int D, int Dv);
 
+extern "C" int64_t jl_attn_scratch_floats(int32_t n_tiles, int32_t n_rows, int32_t H, int32_t Dv, int32_t splits) {
+    return splits > 1 ? (int64_t)n_tiles * splits * H * 32 * 2 + (int64_t)splits * n_rows * H * Dv : 0;
+}
+
 extern "C" int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv) {
     if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0) return 0;
     if (am_fits(dtype, H, G, D, Dv)) return 32;
@@ -218,6 +222,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short am_bf16x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float am_f32x16;
 constexpr int AM_T = 32;
+constexpr int AM_FUSED = 0, AM_STATS = 1, AM_PV = 2;    // both sweeps in one launch; or the keys split over workgroups: statistics, then outputs
 
 __device__ __forceinline__ short am_bf16(float v) {
     uint32_t u = __float_as_uint(v);
@@ -230,7 +235,7 @@ static size_t am_lds_bytes(int H, int G, int D, int Dv) {
 }
 
 template <int HPW, int NDV>
-__global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a) {
+__global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
     const int H = a.H, G = a.G, D = a.D, Dv = a.Dv, rep = H / G, KLD = D + 4;
     const int tid = threadIdx.x, nthr = blockDim.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, hi = lane >> 5;
@@ -251,6 +256,24 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a) {
     const int *bt = a.block_tables + (int64_t)b * a.bt_stride;
     const bf16_t *q = (const bf16_t *)a.q, *kc = (const bf16_t *)a.k_cache, *vc = (const bf16_t *)a.v_cache;
     if (a.talk) for (int e = tid; e < H * H; e += nthr) talk[e] = a.talk[e];
+    // keys split over blockIdx.y (few tiles with many keys: decoding): this workgroup's share of the 32-key tiles
+    const int S = a.splits > 1 ? a.splits : 1, split = blockIdx.y;
+    const int per = ((n_keys + AM_T - 1) / AM_T + S - 1) / S;
+    const int key_lo = split * per * AM_T, key_hi = (split + 1) * per * AM_T < n_keys ? (split + 1) * per * AM_T : n_keys;
+    float *ml = a.scratch;                                          // [tiles][S][H][32][2] maximum, sum of a split
+    float *po = a.scratch + (int64_t)a.n_tiles * S * H * AM_T * 2;  // [S][rows][H * Dv] a split's share of the outputs
+    if (mode == AM_PV) {                                            // join the splits' statistics of this tile
+        for (int e = tid; e < H * AM_T; e += nthr) {
+            float M = -INFINITY, L = 0.f;
+            for (int sp = 0; sp < S; ++sp) M = fmaxf(M, ml[(((int64_t)blockIdx.x * S + sp) * H * AM_T + e) * 2]);
+            for (int sp = 0; sp < S; ++sp) {
+                const float *p2 = ml + (((int64_t)blockIdx.x * S + sp) * H * AM_T + e) * 2;
+                if (p2[0] > -INFINITY) L += p2[1] * __expf(p2[0] - M);
+            }
+            mS[e] = M;
+            lS[e] = L > 0.f ? 1.0f / L : 0.f;
+        }
+    }
 
     float m_run[HPW][16], l_run[HPW][16];
     am_f32x16 acc[HPW][NDV];
@@ -264,9 +287,9 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a) {
             for (int r = 0; r < 16; ++r) acc[x][t][r] = 0.f;
     }
 
-    for (int sweep = 0; sweep < 2; ++sweep) {
-        for (int u0 = 0; u0 < n_keys; u0 += AM_T) {
-            const int nk = n_keys - u0 < AM_T ? n_keys - u0 : AM_T;
+    for (int sweep = (mode == AM_PV ? 1 : 0); sweep < (mode == AM_STATS ? 1 : 2); ++sweep) {
+        for (int u0 = key_lo; u0 < key_hi; u0 += AM_T) {
+            const int nk = key_hi - u0 < AM_T ? key_hi - u0 : AM_T;
             __syncthreads();                                        // the previous tile's readers are done
             const int kq = G * D / 4;                               // 8-byte units per key
             for (int e = tid; e < AM_T * kq; e += nthr) {
@@ -395,10 +418,37 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a) {
 #pragma unroll
                     for (int off = 16; off > 0; off >>= 1) L += __shfl_xor(L, off, 64);
                     const int ii = 8 * (r >> 2) + 4 * hi + (r & 3);
-                    if (l32 == 0 && g < H) { mS[g * AM_T + ii] = M; lS[g * AM_T + ii] = L > 0.f ? 1.0f / L : 0.f; }
+                    if (l32 == 0 && g < H) {
+                        if (mode == AM_STATS) {
+                            float *p2 = ml + ((((int64_t)blockIdx.x * S + split) * H + g) * AM_T + ii) * 2;
+                            p2[0] = M;
+                            p2[1] = L;
+                        } else {
+                            mS[g * AM_T + ii] = M;
+                            lS[g * AM_T + ii] = L > 0.f ? 1.0f / L : 0.f;
+                        }
+                    }
                 }
             }
         }
+    }
+    if (mode == AM_STATS) return;
+    if (mode == AM_PV) {                                            // float shares; attn_join_kernel adds them up and gates
+#pragma unroll
+        for (int x = 0; x < HPW; ++x) {
+            const int h = wave * HPW + x;
+            if (h >= H) continue;
+#pragma unroll
+            for (int t = 0; t < NDV; ++t) {
+                if (32 * t + l32 >= Dv) continue;
+#pragma unroll
+                for (int r = 0; r < 16; ++r) {
+                    const int ii = 8 * (r >> 2) + 4 * hi + (r & 3);
+                    if (ii < cnt) po[((int64_t)split * a.n_rows + row0 + ii) * (H * Dv) + h * Dv + 32 * t + l32] = acc[x][t][r];
+                }
+            }
+        }
+        return;
     }
     bf16_t *out = (bf16_t *)a.out;
     const bf16_t *gate = (const bf16_t *)a.gate;
@@ -422,6 +472,20 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a) {
     }
 }
 
+// out = gate * the sum of the splits' shares, in split order
+__global__ __launch_bounds__(256) void attn_join_kernel(const float *__restrict__ po, int S, int64_t total, int width,
+                                                         const bf16_t *__restrict__ gate, int64_t gate_ld, bf16_t *__restrict__ out) {
+    const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
+    if (e >= total) return;
+    float v = 0.f;
+    for (int sp = 0; sp < S; ++sp) v += po[(int64_t)sp * total + e];
+    if (gate) {
+        const int64_t row = e / width;
+        v *= 1.0f / (1.0f + __expf(-ld_f(gate + row * gate_ld + (e - row * width))));
+    }
+    st_f(out + e, v);
+}
+
 static bool am_fits(int dtype, int H, int G, int D, int Dv) {
     static const bool off = getenv("JL_ATTN_NO_MFMA") != nullptr;          // A/B switch for measurements
     return !off && dtype == JL_BF16 && H <= 16 && D % 8 == 0 && D <= 256 && Dv <= 128 && (G * Dv) % 4 == 0 &&
@@ -436,8 +500,17 @@ template <int HPW, int NDV> static int am_launch(const jl_attn_args &a, hipStrea
         if (e != hipSuccess) return jl_fail(JL_E_LAUNCH, "jl_attn_window: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     }
     const int waves = (a.H + HPW - 1) / HPW;
-    kern<<<dim3((unsigned)a.n_tiles), 64 * waves, lds, st>>>(a);
-    return jl_check_launch("attn_mfma_kernel");
+    if (a.splits <= 1) {
+        kern<<<dim3((unsigned)a.n_tiles), 64 * waves, lds, st>>>(a, AM_FUSED);
+        return jl_check_launch("attn_mfma_kernel");
+    }
+    const dim3 grid((unsigned)a.n_tiles, (unsigned)a.splits);
+    kern<<<grid, 64 * waves, lds, st>>>(a, AM_STATS);
+    kern<<<grid, 64 * waves, lds, st>>>(a, AM_PV);
+    const int64_t total = (int64_t)a.n_rows * a.H * a.Dv;
+    attn_join_kernel<<<dim3((unsigned)((total + 255) / 256)), 256, 0, st>>>(a.scratch + (int64_t)a.n_tiles * a.splits * a.H * AM_T * 2, a.splits, total,
+                                                                          a.H * a.Dv, (const bf16_t *)a.gate, a.gate_ld, (bf16_t *)a.out);
+    return jl_check_launch("attn_mfma_kernel (split keys)");
 }
 
 template <typename T, int ACC> static int att_launch(const jl_attn_args &a, const AttShape &s, hipStream_t st) {
@@ -459,6 +532,8 @@ extern "C" int jl_attn_window(const jl_attn_args *ap, void *stream) {
         return jl_fail(JL_E_INVALID, "jl_attn_window: bad head counts or sizes");
     if ((a.rel != nullptr) != (a.lut != nullptr) || (a.lut && a.lut_len <= 0)) return jl_fail(JL_E_INVALID, "jl_attn_window: rel and lut come together");
     hipStream_t st = (hipStream_t)stream;
+    if (a.splits > 1 && (!a.scratch || a.n_rows <= 0 || !(a.TQ == AM_T && am_fits(a.dtype, a.H, a.G, a.D, a.Dv))))
+        return jl_fail(JL_E_INVALID, "jl_attn_window: split keys need the matrix-core kernel, a scratch and the row count");
     if (a.TQ == AM_T && am_fits(a.dtype, a.H, a.G, a.D, a.Dv)) {
         const int ndv = (a.Dv + 31) / 32;
 #define AM_CASE(HP, ND) if ((a.H > 8 ? 2 : 1) == HP && ndv == ND) return am_launch<HP, ND>(a, st)

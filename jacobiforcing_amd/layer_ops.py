@@ -15,6 +15,7 @@ import torch
 from . import _native as N
 
 
+ATTN_SPLIT_BELOW_TILES, ATTN_SPLIT_WORKGROUPS = 128, 512     # attention: split a tile's keys while tiles x splits stays below ~2 per CU
 RETENTION_CHUNK = 64          # tokens per chunk when a long portion's recurrence is cut into chunks that run side by side
 
 
@@ -195,12 +196,20 @@ def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Te
     tq = attn_tile_rows(dt, H, G, D, Dv)
     tiles = batch.tiles(tq)
     out = torch.empty((n, H * Dv), dtype=dt, device=q.device)
+    # few tiles with many keys (decoding): share each tile's keys out over workgroups until the chip is full
+    splits, scratch = 1, None
+    if tq == 32 and tiles.shape[0] < ATTN_SPLIT_BELOW_TILES:
+        reach = batch.max_pos if window <= 0 else min(batch.max_pos, int(window) + int(keep_first) + tq)
+        splits = max(1, min(-(-reach // 64), ATTN_SPLIT_WORKGROUPS // tiles.shape[0], 64))
+        if splits > 1:
+            scratch = torch.empty((int(N.layers().jl_attn_scratch_floats(tiles.shape[0], n, H, Dv, splits)),), dtype=torch.float32, device=q.device)
     a = N.AttnArgs(q=q.data_ptr(), gate=gate.data_ptr() if gate is not None else None, gate_ld=gate.stride(0) if gate is not None else 0,
                    k_cache=k_cache.data_ptr(), v_cache=v_cache.data_ptr(), out=out.data_ptr(), block_tables=batch.tables.data_ptr(),
                    tiles=tiles.data_ptr(), rel=rel.data_ptr() if rel is not None else None, lut=lut.data_ptr() if rel is not None else None,
                    talk=talk.data_ptr() if talk is not None else None, bt_stride=batch.tables.shape[1], n_tiles=tiles.shape[0],
                    lut_len=lut.numel() if rel is not None else 0, page_size=batch.page_size, H=H, G=G, D=D, Dv=Dv, window=int(window),
-                   keep_first=int(keep_first), TQ=tq, dtype=_code(dt), scale=float(scale))
+                   keep_first=int(keep_first), TQ=tq, dtype=_code(dt), scale=float(scale), splits=splits, n_rows=n,
+                   scratch=scratch.data_ptr() if scratch is not None else None)
     N.check_layers(N.layers().jl_attn_window(C.byref(a), _stream(q.device)), "jl_attn_window")
     return out
 
