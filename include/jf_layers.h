@@ -60,6 +60,7 @@ typedef struct {
     float scale;
     int32_t splits, n_rows;       /* splits > 1 (TQ 32 only): each tile's keys are shared out over `splits` workgroups — statistics, */
     float *scratch;               /* outputs, join: three launches; scratch of jl_attn_scratch_floats() floats, n_rows = N          */
+    void *q_pack;                 /* TQ 32 only: room for n_tiles * 32 * H * D elements (the queries in matrix-operand order)        */
 } jl_attn_args;
 JL_API int64_t jl_attn_scratch_floats(int32_t n_tiles, int32_t n_rows, int32_t H, int32_t Dv, int32_t splits);
 JL_API int jl_attn_window(const jl_attn_args *a, void *stream);

@@ -240,7 +240,7 @@ class AttnArgs(C.Structure):
                 ("block_tables", _vp), ("tiles", _vp), ("rel", _vp), ("lut", _vp), ("talk", _vp),
                 ("bt_stride", _i32), ("n_tiles", _i32), ("lut_len", _i32), ("page_size", _i32), ("H", _i32), ("G", _i32), ("D", _i32),
                 ("Dv", _i32), ("window", _i32), ("keep_first", _i32), ("TQ", _i32), ("dtype", _i32), ("scale", _f32),
-                ("splits", _i32), ("n_rows", _i32), ("scratch", _vp)]
+                ("splits", _i32), ("n_rows", _i32), ("scratch", _vp), ("q_pack", _vp)]
 
 
 _LAYER_SIGNATURES = {

@@ -139,7 +139,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
                     s = dot * a.scale;
                     if (a.rel) {
                         const int n = i - j < a.lut_len ? i - j : a.lut_len - 1;
-                        s += a.rel[a.lut[n] * H + g];
+                        s += a.rel[(a.lut ? a.lut[n] : n) * H + g];
                     }
                 }
                 S[(g * TQ + ii) * TK + jj] = s;
@@ -222,6 +222,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
 typedef __attribute__((__vector_size__(4 * sizeof(short)))) short am_bf16x4;
 typedef __attribute__((__vector_size__(16 * sizeof(float)))) float am_f32x16;
 constexpr int AM_T = 32;
+constexpr int AM_PAGES = 1024;     // page-table entries of a request kept in LDS (longer tables are read from memory)
 constexpr int AM_FUSED = 0, AM_STATS = 1, AM_PV = 2;    // both sweeps in one launch; or the keys split over workgroups: statistics, then outputs
 
 __device__ __forceinline__ short am_bf16(float v) {
@@ -230,32 +231,105 @@ __device__ __forceinline__ short am_bf16(float v) {
     return (short)(u >> 16);
 }
 
+__device__ __forceinline__ void am_load_tile(bf16_t *dst, int dst_row, const bf16_t *src, int src_row, int units, int jj, int r, int dj, int dr,
+                                             int nk, int u0, int kf_end, int lo, const int *bt, int page_size, int page_shift, int tid,
+                                             int nthr) {
+    for (int e0 = tid; e0 < AM_T * units; e0 += 4 * nthr) {
+        uint2 v[4];
+        int off[4];
+#pragma unroll
+        for (int it = 0; it < 4; ++it) {
+            v[it] = make_uint2(0, 0);
+            off[it] = -1;
+            if (e0 + it * nthr < AM_T * units) {
+                off[it] = jj * dst_row + 4 * r;
+                if (jj < nk) {
+                    const int u = u0 + jj, j = u < kf_end ? u : lo + (u - kf_end);
+                    const int pg = page_shift >= 0 ? j >> page_shift : j / page_size;
+                    const int64_t tok = (int64_t)bt[pg] * page_size + (j - pg * page_size);
+                    v[it] = *(const uint2 *)(src + tok * src_row + 4 * r);
+                }
+                jj += dj; r += dr;
+                if (r >= units) { r -= units; ++jj; }
+            }
+        }
+#pragma unroll
+        for (int it = 0; it < 4; ++it)
+            if (off[it] >= 0) *(uint2 *)(dst + off[it]) = v[it];
+    }
+}
+
+// The same loader in two halves, for tiles that are fetched one iteration ahead: am_fetch issues a thread's loads (at most PF of
+// them) into registers, am_stash writes them to LDS once the previous tile's readers are done.  `pages` is the request's page
+// table (in LDS when it fits there).
+constexpr int AM_PF = 4;
+__device__ __forceinline__ void am_fetch(uint2 (&v)[AM_PF], const bf16_t *src, int src_row, int units, int jj, int r, int dj, int dr, int nk,
+                                         int u0, int kf_end, int lo, const int *pages, int page_size, int page_shift, int tid, int nthr) {
+#pragma unroll
+    for (int it = 0; it < AM_PF; ++it) {
+        v[it] = make_uint2(0, 0);
+        if (tid + it * nthr < AM_T * units) {
+            if (jj < nk) {
+                const int u = u0 + jj, j = u < kf_end ? u : lo + (u - kf_end);
+                const int pg = page_shift >= 0 ? j >> page_shift : j / page_size;
+                const int64_t tok = (int64_t)pages[pg] * page_size + (j - pg * page_size);
+                v[it] = *(const uint2 *)(src + tok * src_row + 4 * r);
+            }
+            jj += dj; r += dr;
+            if (r >= units) { r -= units; ++jj; }
+        }
+    }
+}
+__device__ __forceinline__ void am_stash(const uint2 (&v)[AM_PF], bf16_t *dst, int dst_row, int units, int jj, int r, int dj, int dr, int tid,
+                                         int nthr) {
+#pragma unroll
+    for (int it = 0; it < AM_PF; ++it)
+        if (tid + it * nthr < AM_T * units) {
+            *(uint2 *)(dst + jj * dst_row + 4 * r) = v[it];
+            jj += dj; r += dr;
+            if (r >= units) { r -= units; ++jj; }
+        }
+}
+
 static size_t am_lds_bytes(int H, int G, int D, int Dv) {
-    return (size_t)G * AM_T * (D + 4) * 2 + (size_t)AM_T * G * Dv * 2 + ((size_t)H * AM_T * 33 + 2 * (size_t)H * AM_T + (size_t)H * H) * 4;
+    return (size_t)AM_T * (G * D + 4) * 2 + (size_t)AM_T * G * Dv * 2 + ((size_t)H * AM_T * 33 + 2 * (size_t)H * AM_T + (size_t)H * H + (size_t)H * 64 + AM_PAGES) * 4;
 }
 
 template <int HPW, int NDV>
 __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int H = a.H, G = a.G, D = a.D, Dv = a.Dv, rep = H / G, KLD = D + 4;
+    const int H = a.H, G = a.G, D = a.D, Dv = a.Dv, rep = H / G, KROW = G * D + 4;
     const int tid = threadIdx.x, nthr = blockDim.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, hi = lane >> 5;
     const int *tile = a.tiles + 4 * (int64_t)blockIdx.x;
     const int b = tile[0], i0 = tile[1], cnt = tile[2], row0 = tile[3];
     if (b < 0 || cnt <= 0) return;
-    bf16_t *Ks = (bf16_t *)smem;                                   // [G][32][D + 4]
-    bf16_t *Vs = Ks + G * AM_T * KLD;                              // [32][G * Dv]
+    bf16_t *Ks = (bf16_t *)smem;                                   // [32][G * D + 4]
+    bf16_t *Vs = Ks + AM_T * KROW;                                 // [32][G * Dv]
     float *Ps = (float *)(Vs + AM_T * G * Dv);                     // [H][32][33]
     float *mS = Ps + H * AM_T * 33;                                // [H][32] row maximum
     float *lS = mS + H * AM_T;                                     // [H][32] 1 / row sum
     float *talk = lS + H * AM_T;                                   // [H][H]
+    float *biasS = talk + H * H;                                   // [H][64] the distance bias of a key tile: entry ii - jj + 31
+    int *pageS = (int *)(biasS + H * 64);                          // [AM_PAGES] this request's page table up to the tile's last key
     const int window = a.window > 0 ? a.window : 0x3fffffff;
     const int i_max = i0 + cnt - 1;
     const int lo = i0 - window + 1 > 0 ? i0 - window + 1 : 0;
     const int kf_end = a.keep_first < lo ? a.keep_first : lo;
     const int n_keys = kf_end + (i_max + 1 - lo);
     const int *bt = a.block_tables + (int64_t)b * a.bt_stride;
-    const bf16_t *q = (const bf16_t *)a.q, *kc = (const bf16_t *)a.k_cache, *vc = (const bf16_t *)a.v_cache;
+    const bf16_t *kc = (const bf16_t *)a.k_cache, *vc = (const bf16_t *)a.v_cache;
     if (a.talk) for (int e = tid; e < H * H; e += nthr) talk[e] = a.talk[e];
+    const int n_pages = i_max / a.page_size + 1;
+    if (n_pages <= AM_PAGES) {                                      // one trip to memory for the page table instead of one per tile
+        for (int e = tid; e < n_pages; e += nthr) pageS[e] = bt[e];
+        __syncthreads();
+        bt = pageS;
+    }
+    // loaders' starting points and steps (e = tid, tid + nthr, ..: key e / units, unit e % units)
+    const int kq = G * D / 4, vq = G * Dv / 4;
+    const int jj_k0 = tid / kq, r_k0 = tid - jj_k0 * kq, dj_k = nthr / kq, dr_k = nthr - dj_k * kq;
+    const int jj_v0 = tid / vq, r_v0 = tid - jj_v0 * vq, dj_v = nthr / vq, dr_v = nthr - dj_v * vq;
+    const int page_shift = (a.page_size & (a.page_size - 1)) == 0 ? __builtin_ctz(a.page_size) : -1;
     // keys split over blockIdx.y (few tiles with many keys: decoding): this workgroup's share of the 32-key tiles
     const int S = a.splits > 1 ? a.splits : 1, split = blockIdx.y;
     const int per = ((n_keys + AM_T - 1) / AM_T + S - 1) / S;
@@ -287,50 +361,58 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
             for (int r = 0; r < 16; ++r) acc[x][t][r] = 0.f;
     }
 
+    // fetch one tile ahead when a thread's share of a tile fits the registers set aside for it (one head per wavefront only: with
+    // two the accumulators leave no room)
+    const bool ahead = HPW == 1 && AM_T * kq <= AM_PF * nthr && AM_T * vq <= AM_PF * nthr;
+    uint2 pk[AM_PF], pv[AM_PF];
     for (int sweep = (mode == AM_PV ? 1 : 0); sweep < (mode == AM_STATS ? 1 : 2); ++sweep) {
+        if (ahead && key_lo < key_hi) {
+            const int nk0 = key_hi - key_lo < AM_T ? key_hi - key_lo : AM_T;
+            am_fetch(pk, kc, G * D, kq, jj_k0, r_k0, dj_k, dr_k, nk0, key_lo, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+            if (sweep == 1) am_fetch(pv, vc, G * Dv, vq, jj_v0, r_v0, dj_v, dr_v, nk0, key_lo, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+        }
         for (int u0 = key_lo; u0 < key_hi; u0 += AM_T) {
             const int nk = key_hi - u0 < AM_T ? key_hi - u0 : AM_T;
             __syncthreads();                                        // the previous tile's readers are done
-            const int kq = G * D / 4;                               // 8-byte units per key
-            for (int e = tid; e < AM_T * kq; e += nthr) {
-                const int jj = e / kq, r = e - jj * kq, c = r / (D / 4), d4 = r - c * (D / 4);
-                uint2 v = make_uint2(0, 0);
-                if (jj < nk) {
-                    const int u = u0 + jj, j = u < kf_end ? u : lo + (u - kf_end);
-                    const int64_t tok = (int64_t)bt[j / a.page_size] * a.page_size + j % a.page_size;
-                    v = *(const uint2 *)(kc + tok * (G * D) + 4 * r);
-                }
-                *(uint2 *)(Ks + (c * AM_T + jj) * KLD + 4 * d4) = v;
-            }
-            if (sweep == 1) {
-                const int vq = G * Dv / 4;
-                for (int e = tid; e < AM_T * vq; e += nthr) {
-                    const int jj = e / vq, r = e - jj * vq;
-                    uint2 v = make_uint2(0, 0);
-                    if (jj < nk) {
-                        const int u = u0 + jj, j = u < kf_end ? u : lo + (u - kf_end);
-                        const int64_t tok = (int64_t)bt[j / a.page_size] * a.page_size + j % a.page_size;
-                        v = *(const uint2 *)(vc + tok * (G * Dv) + 4 * r);
-                    }
-                    *(uint2 *)(Vs + jj * (G * Dv) + 4 * r) = v;
-                }
+            if (ahead) {                                            // this tile was fetched during the previous one
+                am_stash(pk, Ks, KROW, kq, jj_k0, r_k0, dj_k, dr_k, tid, nthr);
+                if (sweep == 1) am_stash(pv, Vs, G * Dv, vq, jj_v0, r_v0, dj_v, dr_v, tid, nthr);
+            } else {
+                // 8-byte units: thread -> (key jj, unit r of the key's row), stepped without divisions; four loads of a thread are
+                // issued before the first is stored
+                am_load_tile(Ks, KROW, kc, G * D, kq, jj_k0, r_k0, dj_k, dr_k, nk, u0, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+                if (sweep == 1)
+                    am_load_tile(Vs, G * Dv, vc, G * Dv, vq, jj_v0, r_v0, dj_v, dr_v, nk, u0, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
             }
             __syncthreads();
-            // this lane's key (column l32 of the tile)
+            if (ahead && u0 + AM_T < key_hi) {                      // the next tile's rows travel while this one is computed
+                const int nk2 = key_hi - (u0 + AM_T) < AM_T ? key_hi - (u0 + AM_T) : AM_T;
+                am_fetch(pk, kc, G * D, kq, jj_k0, r_k0, dj_k, dr_k, nk2, u0 + AM_T, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+                if (sweep == 1) am_fetch(pv, vc, G * Dv, vq, jj_v0, r_v0, dj_v, dr_v, nk2, u0 + AM_T, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+            }
+            // this lane's key (column l32 of the tile); `straight`: the tile's keys are consecutive positions
             const int u = u0 + l32, j = u < kf_end ? u : lo + (u - kf_end);
+            const bool straight = u0 >= kf_end || u0 + AM_T <= kf_end;
 #pragma unroll
             for (int x = 0; x < HPW; ++x) {
                 const int g = wave * HPW + x;
                 if (g >= H) continue;
                 const int c = g / rep;
+                if (a.rel) {                                        // 63 distances occur in a 32 x 32 tile: one table lookup per lane
+                    const int jt = u0 < kf_end ? u0 : lo + (u0 - kf_end);      // position of the tile's first key (a tile that crosses from
+                    int n = i0 - jt + lane - 31;                                // the kept tokens into the window is handled per element)
+                    n = n < 0 ? 0 : (n < a.lut_len ? n : a.lut_len - 1);
+                    biasS[g * 64 + lane] = a.rel[(a.lut ? a.lut[n] : n) * H + g];
+                }
                 am_f32x16 sc;
 #pragma unroll
                 for (int r = 0; r < 16; ++r) sc[r] = 0.f;
-                const bf16_t *qp = q + (int64_t)(row0 + l32) * (H * D) + g * D + 4 * hi;
-                const bf16_t *kp = Ks + (c * AM_T + l32) * KLD + 4 * hi;
-                for (int kk = 0; kk < D; kk += 8) {
-                    am_bf16x4 qa = {0, 0, 0, 0};
-                    if (l32 < cnt) qa = *(const am_bf16x4 *)(qp + kk);
+                // queries in operand order (attn_pack_q_kernel): a step's 64 lanes read 512 consecutive bytes
+                const am_bf16x4 *qp = (const am_bf16x4 *)a.q_pack + ((int64_t)blockIdx.x * H + g) * (D / 8) * 64 + lane;
+                const bf16_t *kp = Ks + l32 * KROW + c * D + 4 * hi;
+#pragma unroll 8
+                for (int kk = 0; kk < D; kk += 8) {                  // unrolled: the query loads of eight steps are in flight together
+                    const am_bf16x4 qa = qp[(kk >> 3) * 64];
                     const am_bf16x4 kb = *(const am_bf16x4 *)(kp + kk);
                     sc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(qa, kb, sc, 0, 0, 0);
                 }
@@ -342,8 +424,12 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
                     if (ok) {
                         s = sc[r] * a.scale;
                         if (a.rel) {
-                            const int n = i - j < a.lut_len ? i - j : a.lut_len - 1;
-                            s += a.rel[a.lut[n] * H + g];
+                            if (straight) {
+                                s += biasS[g * 64 + ii - l32 + 31];
+                            } else {
+                                const int n = i - j < a.lut_len ? i - j : a.lut_len - 1;
+                                s += a.rel[(a.lut ? a.lut[n] : n) * H + g];
+                            }
                         }
                     }
                     if (sweep == 0) {
@@ -472,6 +558,21 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
     }
 }
 
+// Queries of every tile in the order the A operand wants them: q_pack[tile][head][step][lane] = the four depths 8 step + 4 (lane / 32) ..
+// of row lane % 32 (zeros for rows a tile does not have).  Read straight from [N, H * D], a lane's 8 bytes lie a whole row apart.
+__global__ __launch_bounds__(256) void attn_pack_q_kernel(const bf16_t *__restrict__ q, const int32_t *__restrict__ tiles, int H, int D,
+                                                           uint2 *__restrict__ q_pack) {
+    const int *tile = tiles + 4 * (int64_t)blockIdx.x;
+    const int cnt = tile[2], row0 = tile[3];
+    const int steps = D / 8, per_tile = H * steps * 64;
+    for (int e = threadIdx.x; e < per_tile; e += 256) {
+        const int lane = e & 63, st = (e >> 6) % steps, g = (e >> 6) / steps, l32 = lane & 31, hi = lane >> 5;
+        uint2 v = make_uint2(0, 0);
+        if (l32 < cnt) v = *(const uint2 *)(q + (int64_t)(row0 + l32) * (H * D) + g * D + 8 * st + 4 * hi);
+        q_pack[(int64_t)blockIdx.x * per_tile + e] = v;
+    }
+}
+
 // out = gate * the sum of the splits' shares, in split order
 __global__ __launch_bounds__(256) void attn_join_kernel(const float *__restrict__ po, int S, int64_t total, int width,
                                                          const bf16_t *__restrict__ gate, int64_t gate_ld, bf16_t *__restrict__ out) {
@@ -500,6 +601,7 @@ template <int HPW, int NDV> static int am_launch(const jl_attn_args &a, hipStrea
         if (e != hipSuccess) return jl_fail(JL_E_LAUNCH, "jl_attn_window: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e));
     }
     const int waves = (a.H + HPW - 1) / HPW;
+    attn_pack_q_kernel<<<dim3((unsigned)a.n_tiles), 256, 0, st>>>((const bf16_t *)a.q, a.tiles, a.H, a.D, (uint2 *)a.q_pack);
     if (a.splits <= 1) {
         kern<<<dim3((unsigned)a.n_tiles), 64 * waves, lds, st>>>(a, AM_FUSED);
         return jl_check_launch("attn_mfma_kernel");
@@ -530,11 +632,12 @@ extern "C" int jl_attn_window(const jl_attn_args *ap, void *stream) {
     if (!a.q || !a.k_cache || !a.v_cache || !a.out || !a.block_tables || !a.tiles) return jl_fail(JL_E_INVALID, "jl_attn_window: null pointer");
     if (a.H <= 0 || a.G <= 0 || a.H % a.G || a.D <= 0 || a.Dv <= 0 || a.page_size <= 0 || a.TQ <= 0)
         return jl_fail(JL_E_INVALID, "jl_attn_window: bad head counts or sizes");
-    if ((a.rel != nullptr) != (a.lut != nullptr) || (a.lut && a.lut_len <= 0)) return jl_fail(JL_E_INVALID, "jl_attn_window: rel and lut come together");
+    if ((a.lut && !a.rel) || (a.rel && a.lut_len <= 0)) return jl_fail(JL_E_INVALID, "jl_attn_window: a lut needs rel, and rel needs lut_len");
     hipStream_t st = (hipStream_t)stream;
     if (a.splits > 1 && (!a.scratch || a.n_rows <= 0 || !(a.TQ == AM_T && am_fits(a.dtype, a.H, a.G, a.D, a.Dv))))
         return jl_fail(JL_E_INVALID, "jl_attn_window: split keys need the matrix-core kernel, a scratch and the row count");
     if (a.TQ == AM_T && am_fits(a.dtype, a.H, a.G, a.D, a.Dv)) {
+        if (!a.q_pack) return jl_fail(JL_E_INVALID, "jl_attn_window: the matrix-core kernel needs q_pack (n_tiles * 32 * H * D elements)");
         const int ndv = (a.Dv + 31) / 32;
 #define AM_CASE(HP, ND) if ((a.H > 8 ? 2 : 1) == HP && ndv == ND) return am_launch<HP, ND>(a, st)
         AM_CASE(1, 1); AM_CASE(1, 2); AM_CASE(1, 3); AM_CASE(1, 4);

@@ -125,6 +125,7 @@ def kernel_table(s, prompts, prompt_len, decode_batch, context, dtype=torch.bflo
     rel, talk = torch.randn(16, H, device=dev), torch.eye(H, device=dev)
     from ..modeling.lokizen import distance_bucket_table
     lut = torch.from_numpy(distance_bucket_table(16, 4096, max(prompt_len, context) + 8)).to(dev)
+    rel, lut = rel[lut.long()].contiguous(), None                       # the bias laid out by distance, as the model passes it
     w_up, w_down = rnd(E, ff, W) * 0.02, rnd(E, W, ff) * 0.02
     out = {}
 

@@ -191,8 +191,8 @@ def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Te
     for t, shape in ((rel, None), (talk, (H, H))):
         if t is not None:
             _need(t.dtype == torch.float32 and t.is_contiguous() and (shape is None or tuple(t.shape) == shape), "attn_window: float tables")
-    if rel is not None:
-        _need(lut is not None and lut.dtype == torch.int32 and rel.shape[1] == H, "attn_window: rel [rows, H] with its lut")
+    if rel is not None:                                  # rel [rows, H] with lut [positions] -> row, or rel [positions, H] by distance itself
+        _need(rel.shape[1] == H and (lut is None or lut.dtype == torch.int32), "attn_window: rel [rows, H] (+ int32 lut)")
     tq = attn_tile_rows(dt, H, G, D, Dv)
     tiles = batch.tiles(tq)
     out = torch.empty((n, H * Dv), dtype=dt, device=q.device)
@@ -203,13 +203,15 @@ def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Te
         splits = max(1, min(-(-reach // 64), ATTN_SPLIT_WORKGROUPS // tiles.shape[0], 64))
         if splits > 1:
             scratch = torch.empty((int(N.layers().jl_attn_scratch_floats(tiles.shape[0], n, H, Dv, splits)),), dtype=torch.float32, device=q.device)
+    q_pack = torch.empty((tiles.shape[0] * 32 * H * D,), dtype=dt, device=q.device) if tq == 32 else None
     a = N.AttnArgs(q=q.data_ptr(), gate=gate.data_ptr() if gate is not None else None, gate_ld=gate.stride(0) if gate is not None else 0,
                    k_cache=k_cache.data_ptr(), v_cache=v_cache.data_ptr(), out=out.data_ptr(), block_tables=batch.tables.data_ptr(),
-                   tiles=tiles.data_ptr(), rel=rel.data_ptr() if rel is not None else None, lut=lut.data_ptr() if rel is not None else None,
+                   tiles=tiles.data_ptr(), rel=rel.data_ptr() if rel is not None else None, lut=lut.data_ptr() if lut is not None else None,
                    talk=talk.data_ptr() if talk is not None else None, bt_stride=batch.tables.shape[1], n_tiles=tiles.shape[0],
-                   lut_len=lut.numel() if rel is not None else 0, page_size=batch.page_size, H=H, G=G, D=D, Dv=Dv, window=int(window),
+                   lut_len=(lut.numel() if lut is not None else rel.shape[0]) if rel is not None else 0, page_size=batch.page_size, H=H, G=G, D=D, Dv=Dv, window=int(window),
                    keep_first=int(keep_first), TQ=tq, dtype=_code(dt), scale=float(scale), splits=splits, n_rows=n,
-                   scratch=scratch.data_ptr() if scratch is not None else None)
+                   scratch=scratch.data_ptr() if scratch is not None else None,
+                   q_pack=q_pack.data_ptr() if q_pack is not None else None)
     N.check_layers(N.layers().jl_attn_window(C.byref(a), _stream(q.device)), "jl_attn_window")
     return out
 

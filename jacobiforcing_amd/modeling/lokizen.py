@@ -183,6 +183,9 @@ def random_tensors(cfg: LokizenConfig, seed: int = 0, rel_rows: int = 16) -> Dic
     return t
 
 
+DIRECT_BIAS_POSITIONS = 1 << 16
+
+
 class LokizenModel:
     def __init__(self, cfg: LokizenConfig, weights: LokizenWeights, max_positions: int = 8192):
         self.cfg, self.w = cfg, weights
@@ -215,6 +218,7 @@ class LokizenModel:
         self.max_positions = int(n)
         self._angles.clear()
         self._luts.clear()
+        self._bias = {}
         for i, L in enumerate(self.cfg.layers):
             m = L["mixer"]
             if L["type"] == "retention":
@@ -228,6 +232,8 @@ class LokizenModel:
                 key = (int(self.w.layers[i]["rel"].shape[0]), float(m["bias_max"]))
                 if key not in self._luts:
                     self._luts[key] = torch.from_numpy(distance_bucket_table(key[0], key[1], n)).to(self.device)
+                # up to DIRECT_BIAS_POSITIONS the bias is laid out by distance, [positions, H]: one lookup per score instead of two
+                self._bias[i] = self.w.layers[i]["rel"][self._luts[key].long()].contiguous() if n <= DIRECT_BIAS_POSITIONS else None
 
     # ---- mixers ---------------------------------------------------------------------------------------------------------------
     def _attention(self, run: int, li: int, h: torch.Tensor, batch: LO.RaggedBatch, cache: PagedStateCache) -> torch.Tensor:
@@ -237,8 +243,10 @@ class LokizenModel:
         q = LO.qk_norm_append(proj, w["cols"][:3], H, G, D, Dv, w["q_norm"], w["k_norm"], eps, cache.k[run], cache.v[run], batch.kv_slot)
         gate = proj[:, w["cols"][3]:w["cols"][3] + H * Dv]
         mask = m.get("mask") or {}
+        direct = self._bias.get(li)
+        rel, lut = (direct, None) if direct is not None else (w["rel"], self._luts[(int(w["rel"].shape[0]), float(m["bias_max"]))])
         return LO.attn_window(q, gate, cache.k[run], cache.v[run], batch, H, G, D, Dv, m["scale"], int(mask.get("size", 0)),
-                              int(mask.get("keep_first", 0)), w["rel"], self._luts[(int(w["rel"].shape[0]), float(m["bias_max"]))], w["talk"])
+                              int(mask.get("keep_first", 0)), rel, lut, w["talk"])
 
     def _retention(self, run: int, li: int, h: torch.Tensor, batch: LO.RaggedBatch, cache: PagedStateCache) -> torch.Tensor:
         m, w = self.cfg.layers[li]["mixer"], self.w.layers[li]
