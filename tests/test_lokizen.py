@@ -126,7 +126,7 @@ def test_oracle_mask_and_rotation():
     # scores of rotated q, k depend on the distance only
     q, k = torch.randn(1, 1, 8, dtype=torch.float64), torch.randn(1, 1, 8, dtype=torch.float64)
     rq, rk = O.rotate_half_pairs(q.expand(9, 1, 8), 8, 100.0), O.rotate_half_pairs(k.expand(9, 1, 8), 8, 100.0)
-    assert abs(float((rq[7] * rk[4]).sum() - (rq[5] * rk[2]).sum())) < 1e-9
+    assert abs(float((rq[7] * rk[4]).sum() - (rq[5] * rk[2]).sum())) < 1e-5          # the angles are float32
 
 
 def test_oracle_retention_equals_its_unrolled_sum():

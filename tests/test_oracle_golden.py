@@ -455,7 +455,7 @@ def test_fixtures_regenerate_from_the_reference_byte_for_byte():
     import sys
     from pathlib import Path
     root = Path(__file__).resolve().parents[1]
-    if not Path("/root/reference").is_dir():
+    if not Path("/root/reference").is_dir() or not any(Path("/root/reference").iterdir()):
         pytest.skip("the reference tree is not present here")
     if os.environ.get("JF_SKIP_GOLDEN_CHECK") == "1":
         pytest.skip("JF_SKIP_GOLDEN_CHECK=1")
