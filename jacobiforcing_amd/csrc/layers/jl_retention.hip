@@ -7,8 +7,10 @@
 // sums of squares (unit norm over the head's Dv outputs) are reduced once per group.
 constexpr int RET_TT = 8;
 
-template <typename T, int DMAX>
-__global__ void retention_kernel(const T *__restrict__ proj, int64_t ld, int q_col, int k_col, int v_col, int g_col,
+// MAXT: the largest workgroup the instantiation is launched with.  With 256 the state's DMAX rows stay in registers up to
+// DMAX = 128 (the default bound of 1 024 threads leaves 128 registers per lane and spills them).
+template <typename T, int DMAX, int MAXT>
+__global__ __launch_bounds__(MAXT) void retention_kernel(const T *__restrict__ proj, int64_t ld, int q_col, int k_col, int v_col, int g_col,
                                  const int32_t *__restrict__ seq, int H, int D, int Dv, int rot_dims,
                                  const float *__restrict__ cos_t, const float *__restrict__ sin_t, int64_t table_len,
                                  const float *__restrict__ decay, float eps, float *__restrict__ state, T *__restrict__ out, int mode) {
@@ -98,8 +100,12 @@ static int ret_launch(const void *proj, int64_t ld, int q_col, int k_col, int v_
                       float *state, void *out, int mode, hipStream_t st) {
     const int threads = (Dv + 63) / 64 * 64;
     const size_t lds = (size_t)(2 * RET_TT * D + RET_TT * 16) * 4;
-    retention_kernel<T, DMAX><<<dim3((unsigned)(B * H)), threads, lds, st>>>((const T *)proj, ld, q_col, k_col, v_col, g_col, seq, H, D, Dv,
-                                                                            rot_dims, cos_t, sin_t, table_len, decay, eps, state, (T *)out, mode);
+    if (DMAX >= 128 && threads <= 256)
+        retention_kernel<T, DMAX, 256><<<dim3((unsigned)(B * H)), threads, lds, st>>>((const T *)proj, ld, q_col, k_col, v_col, g_col, seq, H, D, Dv,
+                                                                                     rot_dims, cos_t, sin_t, table_len, decay, eps, state, (T *)out, mode);
+    else
+        retention_kernel<T, DMAX, 1024><<<dim3((unsigned)(B * H)), threads, lds, st>>>((const T *)proj, ld, q_col, k_col, v_col, g_col, seq, H, D, Dv,
+                                                                                      rot_dims, cos_t, sin_t, table_len, decay, eps, state, (T *)out, mode);
     return jl_check_launch("retention_kernel");
 }
 
