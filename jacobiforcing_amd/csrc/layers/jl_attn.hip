@@ -2,6 +2,7 @@
 // distance bias and mixed heads, for prompt portions and single decoded tokens alike (one ragged launch).
 #include "jl_common.h"
 #include <stdlib.h>
+#include <type_traits>
 
 // ---- whole-projection q / k norm + append: one workgroup per token ------------------------------------------------------------
 template <typename T>
@@ -352,20 +353,17 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
     float m_run[HPW][16], l_run[HPW][16];
     am_f32x16 acc[HPW][NDV];
 #pragma unroll
-    for (int x = 0; x < HPW; ++x) {
+    for (int x = 0; x < HPW; ++x)
 #pragma unroll
         for (int r = 0; r < 16; ++r) { m_run[x][r] = -INFINITY; l_run[x][r] = 0.f; }
-#pragma unroll
-        for (int t = 0; t < NDV; ++t)
-#pragma unroll
-            for (int r = 0; r < 16; ++r) acc[x][t][r] = 0.f;
-    }
 
     // fetch one tile ahead when a thread's share of a tile fits the registers set aside for it (one head per wavefront only: with
     // two the accumulators leave no room)
     const bool ahead = HPW == 1 && AM_T * kq <= AM_PF * nthr && AM_T * vq <= AM_PF * nthr;
     uint2 pk[AM_PF], pv[AM_PF];
-    for (int sweep = (mode == AM_PV ? 1 : 0); sweep < (mode == AM_STATS ? 1 : 2); ++sweep) {
+    // one body, instantiated per sweep (the accumulators exist in the second only, the running statistics in the first only)
+    auto run_sweep = [&](auto sweep_c) {
+        constexpr int sweep = decltype(sweep_c)::value;
         if (ahead && key_lo < key_hi) {
             const int nk0 = key_hi - key_lo < AM_T ? key_hi - key_lo : AM_T;
             am_fetch(pk, kc, G * D, kq, jj_k0, r_k0, dj_k, dr_k, nk0, key_lo, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
@@ -410,11 +408,20 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
                 // queries in operand order (attn_pack_q_kernel): a step's 64 lanes read 512 consecutive bytes
                 const am_bf16x4 *qp = (const am_bf16x4 *)a.q_pack + ((int64_t)blockIdx.x * H + g) * (D / 8) * 64 + lane;
                 const bf16_t *kp = Ks + l32 * KROW + c * D + 4 * hi;
+                if constexpr (HPW == 1) {
 #pragma unroll 8
-                for (int kk = 0; kk < D; kk += 8) {                  // unrolled: the query loads of eight steps are in flight together
-                    const am_bf16x4 qa = qp[(kk >> 3) * 64];
-                    const am_bf16x4 kb = *(const am_bf16x4 *)(kp + kk);
-                    sc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(qa, kb, sc, 0, 0, 0);
+                    for (int kk = 0; kk < D; kk += 8) {              // unrolled: the query loads of eight steps are in flight together
+                        const am_bf16x4 qa = qp[(kk >> 3) * 64];
+                        const am_bf16x4 kb = *(const am_bf16x4 *)(kp + kk);
+                        sc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(qa, kb, sc, 0, 0, 0);
+                    }
+                } else {                                             // two heads' accumulators leave room for fewer loads in flight
+#pragma unroll 2
+                    for (int kk = 0; kk < D; kk += 8) {
+                        const am_bf16x4 qa = qp[(kk >> 3) * 64];
+                        const am_bf16x4 kb = *(const am_bf16x4 *)(kp + kk);
+                        sc = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(qa, kb, sc, 0, 0, 0);
+                    }
                 }
 #pragma unroll
                 for (int r = 0; r < 16; ++r) {
@@ -490,7 +497,10 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
                 }
             }
         }
-        if (sweep == 0) {
+    };
+    if (mode != AM_PV) {
+        run_sweep(std::integral_constant<int, 0>{});
+        {
             // merge the lanes' running statistics: rows are shared by the 32 lanes of a half wavefront
 #pragma unroll
             for (int x = 0; x < HPW; ++x) {
@@ -519,6 +529,13 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
         }
     }
     if (mode == AM_STATS) return;
+#pragma unroll
+    for (int x = 0; x < HPW; ++x)
+#pragma unroll
+        for (int t = 0; t < NDV; ++t)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) acc[x][t][r] = 0.f;
+    run_sweep(std::integral_constant<int, 1>{});
     if (mode == AM_PV) {                                            // float shares; attn_join_kernel adds them up and gates
 #pragma unroll
         for (int x = 0; x < HPW; ++x) {
