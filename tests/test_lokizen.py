@@ -400,11 +400,16 @@ def test_long_portions_run_in_chunks(dtype, tol):
 
 
 @gpu
-@pytest.mark.parametrize("H,G,D,Dv", [(12, 4, 64, 128), (8, 2, 128, 64), (3, 1, 24, 40), (16, 16, 32, 32), (5, 5, 8, 100)])
-def test_attention_on_the_matrix_cores(H, G, D, Dv):
-    """bfloat16 attention alone (the MFMA kernel: one or two heads per wavefront, value widths that are no multiple of its
-    32-column tiles) on bfloat16-rounded inputs: two portions that cut a window, then single tokens, pages out of order."""
+@pytest.mark.parametrize("H,G,D,Dv,direct", [(12, 4, 64, 128, True), (8, 2, 128, 64, True), (3, 1, 24, 40, False), (16, 16, 32, 32, True),
+                                               (5, 5, 8, 100, True), (20, 4, 16, 24, True), (4, 2, 12, 20, False)])
+def test_bfloat16_attention_alone(H, G, D, Dv, direct, monkeypatch):
+    """bfloat16 attention alone on bfloat16-rounded inputs: the MFMA kernel (one or two heads per wavefront, value widths that are
+    no multiple of its 32-column tiles) and, for more than 16 heads or a head size that is no multiple of 8, the float-FMA kernel;
+    the bias by distance directly or through the bucket table.  Two portions that cut a window, then single tokens, pages out of
+    order."""
     import torch.nn.functional as F
+    if not direct:
+        monkeypatch.setattr(LK, "DIRECT_BIAS_POSITIONS", 0)
     cfg = make_cfg([dict(attn(heads=H, kv=G, dim=D, vdim=Dv, size=37, keep=5, bias_max=90, scale=D ** -0.5), mlp=None)], width=64, vocab=50)
     rig = Rig(cfg, seed=H, dtype=torch.bfloat16, pages=32)
     T = 110
