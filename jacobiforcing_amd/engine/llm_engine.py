@@ -80,11 +80,15 @@ class LLMEngine:
         items, want = [], []
         for key, tokens, places in entries:
             seq = live.get(key)
+            if seq is None and not tokens:
+                continue
             if seq is None:
                 seq = live[key] = Sequence(list(tokens), SamplingParams(temperature=0.0, max_tokens=1 << 30, ignore_eos=True))
                 self.scheduler.admit(seq)
             else:
                 seq.extend_tokens(tokens)
+            if not tokens:                                      # named in the step without tokens of its own: nothing to run
+                continue
             self.scheduler.reserve(seq, len(tokens))
             items.append((seq, len(tokens)))
             want.append(list(places))

@@ -86,8 +86,11 @@ def distance_bucket_table(rows: int, far: float, length: int) -> np.ndarray:
     big = n >= half
     if big.any():
         f = np.float32
-        step = np.log(n[big].astype(f) / f(half)) / np.log(f(far) / f(half)) * f(rows - half)
-        out[big] = np.minimum(rows - 1, half + np.floor(step).astype(np.int64))
+        with np.errstate(divide="ignore", invalid="ignore"):
+            step = np.log(n[big].astype(f) / f(half)) / np.log(f(far) / f(half)) * f(rows - half)
+        # a table whose far distance is not beyond its half has no logarithmic part: everything from the half on is the last row
+        step = np.nan_to_num(np.floor(step), nan=float(rows), posinf=float(rows), neginf=0.0)
+        out[big] = np.clip(half + step.astype(np.int64), half, rows - 1)
     return out.astype(np.int32)
 
 
