@@ -174,8 +174,10 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__rest
     const int a_row = tid >> 2, a_seg = (tid & 3) * 8;
     const int64_t a_src = rin[a_row] >= 0 ? (int64_t)rin[a_row] * K : -1;
     f32x16_t acc0 = {0}, acc1 = {0};
-    for (int k0 = 0; k0 < K; k0 += MM_TK) {
-        uint4 av = make_uint4(0, 0, 0, 0), bv[2];
+    // a stage's rows travel from memory while the previous stage is multiplied: loaded into registers one iteration ahead
+    uint4 av, bv[2];
+    auto fetch = [&](int k0) {
+        av = make_uint4(0, 0, 0, 0);
         if (a_src >= 0 && k0 + a_seg < K) av = *(const uint4 *)(X + a_src + k0 + a_seg);
 #pragma unroll
         for (int i = 0; i < 2; ++i) {
@@ -183,6 +185,9 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__rest
             bv[i] = make_uint4(0, 0, 0, 0);
             if (n0 + n < n_out && k0 + a_seg < K) bv[i] = *(const uint4 *)(We + (int64_t)(n0 + n) * K + k0 + a_seg);
         }
+    };
+    fetch(0);
+    for (int k0 = 0; k0 < K; k0 += MM_TK) {
         __syncthreads();                                   // the previous stage's readers are done
         {
             uint2 *d = (uint2 *)(As + a_row * MM_LD + a_seg);       // rows are 72 bytes apart: 8-byte stores stay aligned
@@ -196,6 +201,7 @@ __global__ __launch_bounds__(256) void moe_gemm_mfma_kernel(const bf16_t *__rest
             d[1] = make_uint2(bv[i].z, bv[i].w);
         }
         __syncthreads();
+        if (k0 + MM_TK < K) fetch(k0 + MM_TK);
 #pragma unroll
         for (int kk = 0; kk < MM_TK; kk += 8) {
             const int ko = kk + 4 * (lane >> 5);
