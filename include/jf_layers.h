@@ -17,7 +17,7 @@ extern "C" {
 #endif
 
 #define JL_API __attribute__((visibility("default")))
-#define JL_VERSION 100
+#define JL_VERSION 110
 #define JL_OK 0
 #define JL_E_INVALID (-1)
 #define JL_E_LAUNCH (-3)
@@ -61,11 +61,73 @@ typedef struct {
     int32_t splits, n_rows;       /* splits > 1 (TQ 32 only): each tile's keys are shared out over `splits` workgroups — statistics, */
     float *scratch;               /* outputs, join: three launches; scratch of jl_attn_scratch_floats() floats, n_rows = N          */
     void *q_pack;                 /* TQ 32 only: room for n_tiles * 32 * H * D elements (the queries in matrix-operand order)        */
+    /* Pools that are column ranges of wider rows, fewer value heads than key heads, float outputs (all 0 = as described above): */
+    int64_t k_ld, v_ld;           /* row stride of k_cache / v_cache in elements (0: G*D / Gv*Dv).  v_cache may point into k_cache.    */
+    int32_t Gv;                   /* value heads (0: G).  G % Gv == 0; key head c reads value head c % Gv (score maps share values)   */
+    int32_t out_dtype;            /* dtype of `out` when it differs from `dtype`: JL_OUT_F32 = float outputs from bfloat16 inputs     */
 } jl_attn_args;
+#define JL_OUT_SAME 0
+#define JL_OUT_F32 2
 JL_API int64_t jl_attn_scratch_floats(int32_t n_tiles, int32_t n_rows, int32_t H, int32_t Dv, int32_t splits);
 JL_API int jl_attn_window(const jl_attn_args *a, void *stream);
-/* TQ (query rows per tile) the kernel wants for this dtype and these sizes; 0 when they do not fit */
-JL_API int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv);
+/* TQ (query rows per tile) the kernel wants for this dtype, these sizes and these pool row strides (0: dense rows); 0 when
+ * they do not fit */
+JL_API int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv, int64_t k_ld, int64_t v_ld);
+
+/* Sublayer-output norm + residual update: x[n] += y[n] / sqrt(mean(y[n]^2) + eps) * g[0] (x float in place, y of y_dtype, g one
+ * float); when `out` is given, out[n] = x[n] in `out_dtype` (what the next sublayer's product reads). */
+JL_API int jl_norm_add(float *x, const void *y, int y_dtype, const float *g, float eps, void *out, int out_dtype, int64_t N, int32_t W,
+                       void *stream);
+
+/* Polynomial activation with unit-RMS powers: out = c0 n(z) + c1 n(z^2) + c2 n(z^3) + c3, powers element by element,
+ * n(u) = u / sqrt(mean(u^2) + eps) over the row's F values.  z, out [N, F] of `dtype`; coef four floats. */
+JL_API int jl_polynorm(const void *z, int dtype, int64_t N, int32_t F, const float *coef, float eps, void *out, void *stream);
+
+/* Causal depthwise convolution over time, added to its input, with the request's last inputs carried in its slot:
+ *   out[t, c] = x[t, c] + sum_{j < taps} w[c, j] * x[t - taps + 1 + j, c]        (zeros before the sequence's start)
+ * x float [N, W]; w [W, taps] and out [N, W] of `dtype`; row_req [N] int32 the request of every row; seq [B, 4] as above;
+ * tail float [slots, taps - 1, W]: the inputs at positions pos0 - taps + 1 .. pos0 - 1 of the slot's request (entries before
+ * position 0 are never read, so a slot's old content does not matter to a new request).  jl_causal_conv reads the tail;
+ * jl_causal_conv_carry, enqueued after it, moves it to the end of the step's rows.  taps <= JL_CONV_MAX_TAPS. */
+#define JL_CONV_MAX_TAPS 16
+JL_API int jl_causal_conv(const float *x, const void *w, int dtype, const int32_t *row_req, const int32_t *seq, const float *tail,
+                          int64_t N, int32_t W, int32_t taps, void *out, void *stream);
+JL_API int jl_causal_conv_carry(const float *x, const int32_t *seq, int32_t B, float *tail, int32_t W, int32_t taps, void *stream);
+
+/* Per-head query / key norm for attention with M score maps per head, query temperature, cache append.  proj [N, ld] holds q
+ * (H heads x M maps x D at q_col, head by head), k (G x M x D at k_col) and v (G x Dv at v_col).  Every D-vector is RMS-normalised on
+ * its own and multiplied by wq / wk [D]; the query is further multiplied by 1 + t_coef * ln(floor((p + 1) / t_every) + 1), p = pos[n]
+ * (t_coef 0: no temperature).  Queries and keys are written MAP-major — q_out [N, M, H, D], k_cache[slot[n]] = [M, G, D] — so that
+ * query row m*H + h reads key row (m*H + h) / (H/G) = m*G + h/(H/G) and value head (m*G + g) % G: one attention launch with M*H query
+ * heads, M*G key heads and G value heads computes all maps.  v goes to v_cache[slot[n]] as it is. */
+JL_API int jl_head_norm_append(const void *proj, int dtype, int64_t N, int64_t ld, int32_t q_col, int32_t k_col, int32_t v_col, int32_t H,
+                               int32_t G, int32_t M, int32_t D, int32_t Dv, const void *wq, const void *wk, float eps, float t_coef,
+                               int32_t t_every, const int32_t *pos, void *q_out, void *k_cache, void *v_cache, const int64_t *slot,
+                               void *stream);
+
+/* Differential combination of two score maps' outputs: a float [N, 2, H, Dv] (map-major, as the launch above produces);
+ * o = a[0] - lambda * a[1];  out[n, h] = o / sqrt(mean(o^2) + eps) * out_scale over the head's Dv values; out [N, H*Dv] of `dtype`. */
+JL_API int jl_diff_combine(const float *a, int64_t N, int32_t H, int32_t Dv, float lambda, float eps, float out_scale, void *out,
+                           int dtype, void *stream);
+
+/* Latent attention, input side.  proj [N, ld] holds the query latent (Rq columns at q_col) and the key/value latent (R columns at
+ * kv_col) followed by rd rotary key dimensions shared by all heads.
+ *   cq_out [N, Rq] = rms_norm(query latent) * wq
+ *   pool[slot[n]] = [rms_norm(key/value latent) * wkv (R) | rotate(rotary key, pos[n]) (rd)]          (pool rows of R + rd)
+ * rotate: of the first rot_dims dimensions, i and i + rot_dims/2 form a pair (u, v) -> (u cos a - v sin a, v cos a + u sin a),
+ * a from the cos / sin tables [positions, rot_dims/2] float; the rest pass unchanged. */
+JL_API int jl_latent_prep(const void *proj, int dtype, int64_t N, int64_t ld, int32_t q_col, int32_t Rq, int32_t kv_col, int32_t R,
+                          int32_t rd, int32_t rot_dims, const void *wq, const void *wkv, float eps, const int32_t *pos,
+                          const float *cos_t, const float *sin_t, int64_t table_len, void *cq_out, void *pool, const int64_t *slot,
+                          void *stream);
+/* Queries of latent attention in the pool's coordinates: q_out[n, h] = [qa[h, n, :R] | rotate(q[n, h, D : D + rd], pos[n])] with qa
+ * [H, N, R] the unrotated query parts already multiplied by the key up-projection, q [N, H, D + rd]. */
+JL_API int jl_latent_q_pack(const void *qa, const void *q, int dtype, int64_t N, int32_t H, int32_t D, int32_t R, int32_t rd,
+                            int32_t rot_dims, const int32_t *pos, const float *cos_t, const float *sin_t, int64_t table_len, void *q_out,
+                            void *stream);
+/* out[n, h*Dv + d] = ov[h, n, d] * sigmoid(gate[n * gate_ld + h*Dv + d]) (gate null: no gate). */
+JL_API int jl_heads_gate(const void *ov, const void *gate, int64_t gate_ld, int dtype, int64_t N, int32_t H, int32_t Dv, void *out,
+                         void *stream);
 
 /* Retention (linear attention with a fixed decay per head, no denominator) over the ragged batch, state carried in float:
  *   q, k rotated (rotate-half pairs on the first rot_dims dimensions, angles from the cos / sin tables [positions, rot_dims/2]),

@@ -232,6 +232,7 @@ def raise_state_error(code: int, what: str, aux: int = 0):
 # ---- libjf_layers.so (include/jf_layers.h): layer kernels of the models whose forward is not stock PyTorch ----------------------------
 LAYERS_LIB_PATH = _PKG / "lib" / "libjf_layers.so"
 JL_F32, JL_BF16 = 0, 1
+JL_OUT_SAME, JL_OUT_F32 = 0, 2
 
 
 class AttnArgs(C.Structure):
@@ -240,7 +241,8 @@ class AttnArgs(C.Structure):
                 ("block_tables", _vp), ("tiles", _vp), ("rel", _vp), ("lut", _vp), ("talk", _vp),
                 ("bt_stride", _i32), ("n_tiles", _i32), ("lut_len", _i32), ("page_size", _i32), ("H", _i32), ("G", _i32), ("D", _i32),
                 ("Dv", _i32), ("window", _i32), ("keep_first", _i32), ("TQ", _i32), ("dtype", _i32), ("scale", _f32),
-                ("splits", _i32), ("n_rows", _i32), ("scratch", _vp), ("q_pack", _vp)]
+                ("splits", _i32), ("n_rows", _i32), ("scratch", _vp), ("q_pack", _vp), ("k_ld", _i64), ("v_ld", _i64), ("Gv", _i32),
+                ("out_dtype", _i32)]
 
 
 _LAYER_SIGNATURES = {
@@ -251,7 +253,18 @@ _LAYER_SIGNATURES = {
     "jl_qk_norm_append": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _vp, _vp, _vp, _vp, _vp]),
     "jl_attn_window": (C.c_int, [C.POINTER(AttnArgs), _vp]),
     "jl_attn_scratch_floats": (_i64, [_i32, _i32, _i32, _i32, _i32]),
-    "jl_attn_tile_rows": (C.c_int, [C.c_int, _i32, _i32, _i32, _i32]),
+    "jl_attn_tile_rows": (C.c_int, [C.c_int, _i32, _i32, _i32, _i32, _i64, _i64]),
+    "jl_norm_add": (C.c_int, [_vp, _vp, C.c_int, _vp, _f32, _vp, C.c_int, _i64, _i32, _vp]),
+    "jl_polynorm": (C.c_int, [_vp, C.c_int, _i64, _i32, _vp, _f32, _vp, _vp]),
+    "jl_causal_conv": (C.c_int, [_vp, _vp, C.c_int, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _vp]),
+    "jl_causal_conv_carry": (C.c_int, [_vp, _vp, _i32, _vp, _i32, _i32, _vp]),
+    "jl_head_norm_append": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _f32, _i32,
+                                      _vp, _vp, _vp, _vp, _vp, _vp]),
+    "jl_diff_combine": (C.c_int, [_vp, _i64, _i32, _i32, _f32, _f32, _f32, _vp, C.c_int, _vp]),
+    "jl_latent_prep": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _vp, _vp,
+                                 _vp, _vp]),
+    "jl_latent_q_pack": (C.c_int, [_vp, _vp, C.c_int, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp, _vp]),
+    "jl_heads_gate": (C.c_int, [_vp, _vp, _i64, C.c_int, _i64, _i32, _i32, _vp, _vp]),
     "jl_retention": (C.c_int, [_vp, C.c_int, _i64, _i32, _i32, _i32, _i32, _vp, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _i64, _vp, _f32,
                                _vp, _vp, _i32, _vp]),
     "jl_retention_join": (C.c_int, [_vp, _i32, _vp, _i32, _i32, _i32, _vp, _vp, _vp, _vp]),

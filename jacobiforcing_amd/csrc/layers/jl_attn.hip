@@ -71,14 +71,16 @@ static bool att_shape(int H, int G, int D, int Dv, int tq_want, AttShape *o) {
 }
 
 static bool am_fits(int dtype, int H, int G, int D, int Dv);
+// the matrix-core kernel loads pool rows in 8-byte units: row strides must be multiples of four elements
+static bool am_strides_ok(int64_t k_ld, int64_t v_ld) { return k_ld % 4 == 0 && v_ld % 4 == 0; }
 
 extern "C" int64_t jl_attn_scratch_floats(int32_t n_tiles, int32_t n_rows, int32_t H, int32_t Dv, int32_t splits) {
     return splits > 1 ? (int64_t)n_tiles * splits * H * 32 * 2 + (int64_t)splits * n_rows * H * Dv : 0;
 }
 
-extern "C" int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv) {
+extern "C" int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv, int64_t k_ld, int64_t v_ld) {
     if (H <= 0 || G <= 0 || H % G || D <= 0 || Dv <= 0) return 0;
-    if (am_fits(dtype, H, G, D, Dv)) return 32;
+    if (am_fits(dtype, H, G, D, Dv) && am_strides_ok(k_ld, v_ld)) return 32;
     AttShape s;
     return att_shape(H, G, D, Dv, 0, &s) ? s.TQ : 0;
 }
@@ -86,7 +88,7 @@ extern "C" int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int
 template <typename T, int ACC>
 __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a, int TK) {
     extern __shared__ float lds[];
-    const int H = a.H, G = a.G, D = a.D, Dv = a.Dv, TQ = a.TQ, rep = H / G;
+    const int H = a.H, G = a.G, D = a.D, Dv = a.Dv, TQ = a.TQ, rep = H / G, Gv = a.Gv;
     const int tid = threadIdx.x;
     const int *tile = a.tiles + 4 * (int64_t)blockIdx.x;
     const int b = tile[0], i0 = tile[1], cnt = tile[2], row0 = tile[3];
@@ -126,7 +128,7 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
                 const int jj = e / (G * D), r = e - jj * (G * D), c = r / D, d = r - c * D;
                 const int u = u0 + jj, j = u < kf_end ? u : lo + (u - kf_end);
                 const int64_t tok = (int64_t)bt[j / a.page_size] * a.page_size + j % a.page_size;
-                KV[(c * TK + jj) * kstride + d] = ld_f(kc + tok * (G * D) + r);
+                KV[(c * TK + jj) * kstride + d] = ld_f(kc + tok * a.k_ld + r);
             }
             __syncthreads();
             for (int e = tid; e < H * cnt * nk; e += ATT_THREADS) {
@@ -166,11 +168,11 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
                 const int o = (g * TQ + ii) * TK + jj;
                 S[o] = expf(S[o] - mx[g * TQ + ii]) / sm[g * TQ + ii];
             }
-            for (int e = tid; e < nk * G * Dv; e += ATT_THREADS) {   // keys are no longer read: the values take their place
-                const int jj = e / (G * Dv), r = e - jj * (G * Dv);
+            for (int e = tid; e < nk * Gv * Dv; e += ATT_THREADS) {  // keys are no longer read: the values take their place
+                const int jj = e / (Gv * Dv), r = e - jj * (Gv * Dv);
                 const int u = u0 + jj, j = u < kf_end ? u : lo + (u - kf_end);
                 const int64_t tok = (int64_t)bt[j / a.page_size] * a.page_size + j % a.page_size;
-                KV[jj * (G * Dv) + r] = ld_f(vc + tok * (G * Dv) + r);
+                KV[jj * (Gv * Dv) + r] = ld_f(vc + tok * a.v_ld + r);
             }
             __syncthreads();
             const float *Wp = S;
@@ -189,9 +191,9 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
                 const int e = x * ATT_THREADS + tid;
                 if (e < cnt * H * Dv) {
                     const int ii = e / (H * Dv), r = e - ii * (H * Dv), h = r / Dv, d = r - h * Dv;
-                    const float *wp = Wp + (h * TQ + ii) * TK, *vp = KV + (h / rep) * Dv + d;
+                    const float *wp = Wp + (h * TQ + ii) * TK, *vp = KV + ((h / rep) % Gv) * Dv + d;
                     float s = acc[x];
-                    for (int jj = 0; jj < nk; ++jj) s += wp[jj] * vp[jj * (G * Dv)];
+                    for (int jj = 0; jj < nk; ++jj) s += wp[jj] * vp[jj * (Gv * Dv)];
                     acc[x] = s;
                 }
             }
@@ -206,7 +208,8 @@ __global__ __launch_bounds__(ATT_THREADS) void attn_window_kernel(jl_attn_args a
             const int ii = e / (H * Dv), r = e - ii * (H * Dv);
             float v = acc[x];
             if (gate) v *= 1.0f / (1.0f + expf(-ld_f(gate + (int64_t)(row0 + ii) * a.gate_ld + r)));
-            st_f(out + (int64_t)(row0 + ii) * (H * Dv) + r, v);
+            if (a.out_dtype == JL_OUT_F32) ((float *)a.out)[(int64_t)(row0 + ii) * (H * Dv) + r] = v;
+            else st_f(out + (int64_t)(row0 + ii) * (H * Dv) + r, v);
         }
     }
 }
@@ -299,13 +302,13 @@ static size_t am_lds_bytes(int H, int G, int D, int Dv) {
 template <int HPW, int NDV>
 __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int H = a.H, G = a.G, D = a.D, Dv = a.Dv, rep = H / G, KROW = G * D + 4;
+    const int H = a.H, G = a.G, D = a.D, Dv = a.Dv, rep = H / G, KROW = G * D + 4, Gv = a.Gv, VROW = Gv * Dv;
     const int tid = threadIdx.x, nthr = blockDim.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, hi = lane >> 5;
     const int *tile = a.tiles + 4 * (int64_t)blockIdx.x;
     const int b = tile[0], i0 = tile[1], cnt = tile[2], row0 = tile[3];
     if (b < 0 || cnt <= 0) return;
     bf16_t *Ks = (bf16_t *)smem;                                   // [32][G * D + 4]
-    bf16_t *Vs = Ks + AM_T * KROW;                                 // [32][G * Dv]
+    bf16_t *Vs = Ks + AM_T * KROW;                                 // [32][Gv * Dv] (room for G * Dv)
     float *Ps = (float *)(Vs + AM_T * G * Dv);                     // [H][32][33]
     float *mS = Ps + H * AM_T * 33;                                // [H][32] row maximum
     float *lS = mS + H * AM_T;                                     // [H][32] 1 / row sum
@@ -327,7 +330,7 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
         bt = pageS;
     }
     // loaders' starting points and steps (e = tid, tid + nthr, ..: key e / units, unit e % units)
-    const int kq = G * D / 4, vq = G * Dv / 4;
+    const int kq = G * D / 4, vq = VROW / 4;
     const int jj_k0 = tid / kq, r_k0 = tid - jj_k0 * kq, dj_k = nthr / kq, dr_k = nthr - dj_k * kq;
     const int jj_v0 = tid / vq, r_v0 = tid - jj_v0 * vq, dj_v = nthr / vq, dr_v = nthr - dj_v * vq;
     const int page_shift = (a.page_size & (a.page_size - 1)) == 0 ? __builtin_ctz(a.page_size) : -1;
@@ -366,27 +369,27 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
         constexpr int sweep = decltype(sweep_c)::value;
         if (ahead && key_lo < key_hi) {
             const int nk0 = key_hi - key_lo < AM_T ? key_hi - key_lo : AM_T;
-            am_fetch(pk, kc, G * D, kq, jj_k0, r_k0, dj_k, dr_k, nk0, key_lo, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
-            if (sweep == 1) am_fetch(pv, vc, G * Dv, vq, jj_v0, r_v0, dj_v, dr_v, nk0, key_lo, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+            am_fetch(pk, kc, a.k_ld, kq, jj_k0, r_k0, dj_k, dr_k, nk0, key_lo, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+            if (sweep == 1) am_fetch(pv, vc, a.v_ld, vq, jj_v0, r_v0, dj_v, dr_v, nk0, key_lo, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
         }
         for (int u0 = key_lo; u0 < key_hi; u0 += AM_T) {
             const int nk = key_hi - u0 < AM_T ? key_hi - u0 : AM_T;
             __syncthreads();                                        // the previous tile's readers are done
             if (ahead) {                                            // this tile was fetched during the previous one
                 am_stash(pk, Ks, KROW, kq, jj_k0, r_k0, dj_k, dr_k, tid, nthr);
-                if (sweep == 1) am_stash(pv, Vs, G * Dv, vq, jj_v0, r_v0, dj_v, dr_v, tid, nthr);
+                if (sweep == 1) am_stash(pv, Vs, VROW, vq, jj_v0, r_v0, dj_v, dr_v, tid, nthr);
             } else {
                 // 8-byte units: thread -> (key jj, unit r of the key's row), stepped without divisions; four loads of a thread are
                 // issued before the first is stored
-                am_load_tile(Ks, KROW, kc, G * D, kq, jj_k0, r_k0, dj_k, dr_k, nk, u0, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+                am_load_tile(Ks, KROW, kc, a.k_ld, kq, jj_k0, r_k0, dj_k, dr_k, nk, u0, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
                 if (sweep == 1)
-                    am_load_tile(Vs, G * Dv, vc, G * Dv, vq, jj_v0, r_v0, dj_v, dr_v, nk, u0, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+                    am_load_tile(Vs, VROW, vc, a.v_ld, vq, jj_v0, r_v0, dj_v, dr_v, nk, u0, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
             }
             __syncthreads();
             if (ahead && u0 + AM_T < key_hi) {                      // the next tile's rows travel while this one is computed
                 const int nk2 = key_hi - (u0 + AM_T) < AM_T ? key_hi - (u0 + AM_T) : AM_T;
-                am_fetch(pk, kc, G * D, kq, jj_k0, r_k0, dj_k, dr_k, nk2, u0 + AM_T, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
-                if (sweep == 1) am_fetch(pv, vc, G * Dv, vq, jj_v0, r_v0, dj_v, dr_v, nk2, u0 + AM_T, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+                am_fetch(pk, kc, a.k_ld, kq, jj_k0, r_k0, dj_k, dr_k, nk2, u0 + AM_T, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
+                if (sweep == 1) am_fetch(pv, vc, a.v_ld, vq, jj_v0, r_v0, dj_v, dr_v, nk2, u0 + AM_T, kf_end, lo, bt, a.page_size, page_shift, tid, nthr);
             }
             // this lane's key (column l32 of the tile); `straight`: the tile's keys are consecutive positions
             const int u = u0 + l32, j = u < kf_end ? u : lo + (u - kf_end);
@@ -485,13 +488,13 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
                 for (int x = 0; x < HPW; ++x) {
                     const int h = wave * HPW + x;
                     if (h >= H) continue;
-                    const int c = h / rep;
+                    const int c = (h / rep) % Gv;
                     const am_bf16x4 wa = {am_bf16(w[x][0]), am_bf16(w[x][1]), am_bf16(w[x][2]), am_bf16(w[x][3])};
 #pragma unroll
                     for (int t = 0; t < NDV; ++t) {
                         if (32 * t >= Dv) continue;
-                        const bf16_t *vp = Vs + j0 * (G * Dv) + c * Dv + 32 * t + l32;
-                        const am_bf16x4 vb = {(short)vp[0], (short)vp[G * Dv], (short)vp[2 * G * Dv], (short)vp[3 * G * Dv]};
+                        const bf16_t *vp = Vs + j0 * VROW + c * Dv + 32 * t + l32;
+                        const am_bf16x4 vb = {(short)vp[0], (short)vp[VROW], (short)vp[2 * VROW], (short)vp[3 * VROW]};
                         acc[x][t] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(wa, vb, acc[x][t], 0, 0, 0);
                     }
                 }
@@ -569,7 +572,8 @@ __global__ __launch_bounds__(512) void attn_mfma_kernel(jl_attn_args a, int mode
                 const int col = h * Dv + 32 * t + l32;
                 float v = acc[x][t][r];
                 if (gate) v *= 1.0f / (1.0f + __expf(-ld_f(gate + (int64_t)(row0 + ii) * a.gate_ld + col)));
-                st_f(out + (int64_t)(row0 + ii) * (H * Dv) + col, v);
+                if (a.out_dtype == JL_OUT_F32) ((float *)a.out)[(int64_t)(row0 + ii) * (H * Dv) + col] = v;
+                else st_f(out + (int64_t)(row0 + ii) * (H * Dv) + col, v);
             }
         }
     }
@@ -592,7 +596,7 @@ __global__ __launch_bounds__(256) void attn_pack_q_kernel(const bf16_t *__restri
 
 // out = gate * the sum of the splits' shares, in split order
 __global__ __launch_bounds__(256) void attn_join_kernel(const float *__restrict__ po, int S, int64_t total, int width,
-                                                         const bf16_t *__restrict__ gate, int64_t gate_ld, bf16_t *__restrict__ out) {
+                                                         const bf16_t *__restrict__ gate, int64_t gate_ld, bf16_t *__restrict__ out, int out_f32) {
     const int64_t e = (int64_t)blockIdx.x * 256 + threadIdx.x;
     if (e >= total) return;
     float v = 0.f;
@@ -601,12 +605,13 @@ __global__ __launch_bounds__(256) void attn_join_kernel(const float *__restrict_
         const int64_t row = e / width;
         v *= 1.0f / (1.0f + __expf(-ld_f(gate + row * gate_ld + (e - row * width))));
     }
-    st_f(out + e, v);
+    if (out_f32) ((float *)out)[e] = v;
+    else st_f(out + e, v);
 }
 
 static bool am_fits(int dtype, int H, int G, int D, int Dv) {
     static const bool off = getenv("JL_ATTN_NO_MFMA") != nullptr;          // A/B switch for measurements
-    return !off && dtype == JL_BF16 && H <= 16 && D % 8 == 0 && D <= 256 && Dv <= 128 && (G * Dv) % 4 == 0 &&
+    return !off && dtype == JL_BF16 && H <= 16 && D % 8 == 0 && D <= 256 && Dv <= 128 && Dv % 4 == 0 &&
            am_lds_bytes(H, G, D, Dv) <= (size_t)ATT_LDS_BUDGET + 8 * 1024;
 }
 
@@ -628,7 +633,7 @@ template <int HPW, int NDV> static int am_launch(const jl_attn_args &a, hipStrea
     kern<<<grid, 64 * waves, lds, st>>>(a, AM_PV);
     const int64_t total = (int64_t)a.n_rows * a.H * a.Dv;
     attn_join_kernel<<<dim3((unsigned)((total + 255) / 256)), 256, 0, st>>>(a.scratch + (int64_t)a.n_tiles * a.splits * a.H * AM_T * 2, a.splits, total,
-                                                                          a.H * a.Dv, (const bf16_t *)a.gate, a.gate_ld, (bf16_t *)a.out);
+                                                                          a.H * a.Dv, (const bf16_t *)a.gate, a.gate_ld, (bf16_t *)a.out, a.out_dtype == JL_OUT_F32);
     return jl_check_launch("attn_mfma_kernel (split keys)");
 }
 
@@ -650,10 +655,17 @@ extern "C" int jl_attn_window(const jl_attn_args *ap, void *stream) {
     if (a.H <= 0 || a.G <= 0 || a.H % a.G || a.D <= 0 || a.Dv <= 0 || a.page_size <= 0 || a.TQ <= 0)
         return jl_fail(JL_E_INVALID, "jl_attn_window: bad head counts or sizes");
     if ((a.lut && !a.rel) || (a.rel && a.lut_len <= 0)) return jl_fail(JL_E_INVALID, "jl_attn_window: a lut needs rel, and rel needs lut_len");
+    if (a.Gv <= 0) a.Gv = a.G;
+    if (a.k_ld <= 0) a.k_ld = (int64_t)a.G * a.D;
+    if (a.v_ld <= 0) a.v_ld = (int64_t)a.Gv * a.Dv;
+    if (a.G % a.Gv || a.k_ld < (int64_t)a.G * a.D || a.v_ld < (int64_t)a.Gv * a.Dv)
+        return jl_fail(JL_E_INVALID, "jl_attn_window: value heads must divide the key heads, and row strides hold a row");
+    if (a.out_dtype != JL_OUT_SAME && a.out_dtype != JL_OUT_F32) return jl_fail(JL_E_INVALID, "jl_attn_window: unknown out_dtype");
+    if (a.dtype == JL_F32) a.out_dtype = JL_OUT_SAME;
     hipStream_t st = (hipStream_t)stream;
-    if (a.splits > 1 && (!a.scratch || a.n_rows <= 0 || !(a.TQ == AM_T && am_fits(a.dtype, a.H, a.G, a.D, a.Dv))))
+    if (a.splits > 1 && (!a.scratch || a.n_rows <= 0 || !(a.TQ == AM_T && am_fits(a.dtype, a.H, a.G, a.D, a.Dv) && am_strides_ok(a.k_ld, a.v_ld))))
         return jl_fail(JL_E_INVALID, "jl_attn_window: split keys need the matrix-core kernel, a scratch and the row count");
-    if (a.TQ == AM_T && am_fits(a.dtype, a.H, a.G, a.D, a.Dv)) {
+    if (a.TQ == AM_T && am_fits(a.dtype, a.H, a.G, a.D, a.Dv) && am_strides_ok(a.k_ld, a.v_ld)) {
         if (!a.q_pack) return jl_fail(JL_E_INVALID, "jl_attn_window: the matrix-core kernel needs q_pack (n_tiles * 32 * H * D elements)");
         const int ndv = (a.Dv + 31) / 32;
 #define AM_CASE(HP, ND) if ((a.H > 8 ? 2 : 1) == HP && ndv == ND) return am_launch<HP, ND>(a, st)

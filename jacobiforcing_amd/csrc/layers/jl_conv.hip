@@ -1,0 +1,66 @@
+// jl_conv.hip — causal depthwise convolution over time on the float residual stream, added to its input, with the last inputs of
+// every request carried in its state slot (so a prompt may be cut anywhere and decoding continues token by token).
+#include "jl_common.h"
+
+// one workgroup per row; a thread per channel.  Input t - taps + 1 + j of the request comes from the step's own rows when it is
+// one of them, from the slot's tail when it lies before the step, and is zero before the sequence's start.
+template <typename T>
+__global__ __launch_bounds__(256) void causal_conv_kernel(const float *__restrict__ x, const T *__restrict__ w, const int32_t *__restrict__ row_req,
+                                                           const int32_t *__restrict__ seq, const float *__restrict__ tail, int W, int taps,
+                                                           T *__restrict__ out) {
+    const int64_t n = blockIdx.x;
+    const int32_t *rec = seq + 4 * (int64_t)row_req[n];
+    const int row0 = rec[0], pos0 = rec[2], slot = rec[3];
+    const int t = (int)(n - row0), keep = taps - 1;
+    for (int c = threadIdx.x; c < W; c += 256) {
+        float acc = x[n * W + c];
+        for (int j = 0; j < taps; ++j) {
+            const int u = t - keep + j;                         // index among the step's rows of this request
+            float v = 0.f;
+            if (u >= 0) v = x[(int64_t)(row0 + u) * W + c];
+            else if (pos0 + u >= 0) v = tail[((int64_t)slot * keep + (keep + u)) * W + c];
+            acc += ld_f(w + (int64_t)c * taps + j) * v;
+        }
+        st_f(out + n * W + c, acc);
+    }
+}
+
+extern "C" int jl_causal_conv(const float *x, const void *w, int dtype, const int32_t *row_req, const int32_t *seq, const float *tail,
+                              int64_t N, int32_t W, int32_t taps, void *out, void *stream) {
+    if (N <= 0) return JL_OK;
+    if (!x || !w || !row_req || !seq || !out || W <= 0 || taps < 1 || taps > JL_CONV_MAX_TAPS || (taps > 1 && !tail))
+        return jl_fail(JL_E_INVALID, "jl_causal_conv: null pointer, bad width or taps outside 1..%d", JL_CONV_MAX_TAPS);
+    JL_DISPATCH(dtype, causal_conv_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(x, (const T *)w, row_req, seq, tail, W, taps,
+                                                                                                  (T *)out));
+    return jl_check_launch("causal_conv_kernel");
+}
+
+// the tail after the step: the last taps - 1 inputs up to the step's last row.  A thread owns a channel of a request: it reads
+// everything it needs before it writes.
+__global__ __launch_bounds__(256) void causal_conv_carry_kernel(const float *__restrict__ x, const int32_t *__restrict__ seq,
+                                                                 float *__restrict__ tail, int W, int taps) {
+    const int32_t *rec = seq + 4 * (int64_t)blockIdx.y;
+    const int row0 = rec[0], count = rec[1], pos0 = rec[2], slot = rec[3], keep = taps - 1;
+    const int c = blockIdx.x * 256 + threadIdx.x;
+    if (c >= W || count <= 0) return;
+    float v[JL_CONV_MAX_TAPS];
+#pragma unroll
+    for (int s = 0; s < JL_CONV_MAX_TAPS - 1; ++s) {
+        v[s] = 0.f;
+        if (s < keep) {
+            const int u = count - keep + s;
+            if (u >= 0) v[s] = x[(int64_t)(row0 + u) * W + c];
+            else if (pos0 + u >= 0) v[s] = tail[((int64_t)slot * keep + (keep + u)) * W + c];
+        }
+    }
+#pragma unroll
+    for (int s = 0; s < JL_CONV_MAX_TAPS - 1; ++s)
+        if (s < keep) tail[((int64_t)slot * keep + s) * W + c] = v[s];
+}
+
+extern "C" int jl_causal_conv_carry(const float *x, const int32_t *seq, int32_t B, float *tail, int32_t W, int32_t taps, void *stream) {
+    if (B <= 0 || taps <= 1) return JL_OK;
+    if (!x || !seq || !tail || W <= 0 || taps > JL_CONV_MAX_TAPS) return jl_fail(JL_E_INVALID, "jl_causal_conv_carry: null pointer or bad sizes");
+    causal_conv_carry_kernel<<<dim3((unsigned)((W + 255) / 256), (unsigned)B), 256, 0, (hipStream_t)stream>>>(x, seq, tail, W, taps);
+    return jl_check_launch("causal_conv_carry_kernel");
+}

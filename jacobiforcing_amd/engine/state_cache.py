@@ -15,11 +15,14 @@ import torch
 @dataclass
 class RunSpec:
     """Memory one layer run needs.  kind "kv": ``k_width`` / ``v_width`` elements per cached token (all key/value heads side by
-    side).  kind "state": a float tensor of ``state_shape`` per slot.  kind None: nothing."""
+    side; ``v_width`` 0: the values are read out of the key rows, there is no second pool).  kind "state": a float tensor of
+    ``state_shape`` per slot.  kind None: nothing.  Beside either, ``tail_shape`` (when not empty) is a small float tensor per slot
+    for what a layer carries from step to step whatever its mixer is (the last inputs of a short convolution)."""
     kind: Optional[str]
     k_width: int = 0
     v_width: int = 0
     state_shape: tuple = ()
+    tail_shape: tuple = ()
 
 
 class PagedStateCache:
@@ -30,11 +33,14 @@ class PagedStateCache:
         self.k: List[Optional[torch.Tensor]] = []
         self.v: List[Optional[torch.Tensor]] = []
         self.state: List[Optional[torch.Tensor]] = []
+        self.tail: List[Optional[torch.Tensor]] = []
         for s in specs:
             kv = s.kind == "kv"
             self.k.append(torch.zeros((tokens, s.k_width), dtype=dtype, device=device) if kv else None)
-            self.v.append(torch.zeros((tokens, s.v_width), dtype=dtype, device=device) if kv else None)
+            self.v.append(torch.zeros((tokens, s.v_width), dtype=dtype, device=device) if kv and s.v_width else None)
+            self.tail.append(torch.zeros((self.num_slots, *s.tail_shape), dtype=torch.float32, device=device)
+                             if s.tail_shape and all(int(d) > 0 for d in s.tail_shape) else None)
             self.state.append(torch.zeros((self.num_slots, *s.state_shape), dtype=torch.float32, device=device) if s.kind == "state" else None)
 
     def bytes(self) -> int:
-        return sum(t.numel() * t.element_size() for ts in (self.k, self.v, self.state) for t in ts if t is not None)
+        return sum(t.numel() * t.element_size() for ts in (self.k, self.v, self.state, self.tail) for t in ts if t is not None)

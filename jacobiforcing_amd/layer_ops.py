@@ -49,7 +49,7 @@ def _dev(t: torch.Tensor) -> None:
 class RaggedBatch:
     """What one step runs: requests b = 0..B-1 with ``counts[b]`` new tokens from position ``starts[b]``, state slot ``slots[b]``
     and pages ``block_tables[b]``.  Device tensors: ``seq`` [B, 4] int32 {row0, count, pos0, slot}, ``kv_slot`` [N] int64 (pool
-    token of every new row), ``tables`` [B, C] int32."""
+    token of every new row), ``tables`` [B, C] int32, ``row_req`` / ``pos`` [N] int32 (request and position of every row)."""
     B: int
     N: int
     counts: List[int]
@@ -57,6 +57,8 @@ class RaggedBatch:
     seq: torch.Tensor
     kv_slot: torch.Tensor
     tables: torch.Tensor
+    row_req: torch.Tensor
+    pos: torch.Tensor
     page_size: int
     max_pos: int
     max_page: int
@@ -72,6 +74,7 @@ class RaggedBatch:
         C_ = max(1, max(len(t) for t in block_tables))
         bt = np.full((B, C_), -1, dtype=np.int32)
         kv = np.empty(int(row0[-1]), dtype=np.int64)
+        row_pos = np.empty(int(row0[-1]), dtype=np.int32)
         for b in range(B):
             t = np.asarray(block_tables[b], dtype=np.int64)
             bt[b, :t.size] = t
@@ -79,9 +82,12 @@ class RaggedBatch:
             if counts[b] and (starts[b] + counts[b] + page_size - 1) // page_size > t.size:
                 raise ValueError(f"request {b}: {t.size} pages do not hold {starts[b] + counts[b]} tokens")
             kv[row0[b]:row0[b + 1]] = t[pos // page_size] * page_size + pos % page_size
+            row_pos[row0[b]:row0[b + 1]] = pos
         dev = torch.device(device)
         return cls(B=B, N=int(row0[-1]), counts=list(map(int, counts)), starts=list(map(int, starts)),
                    seq=torch.from_numpy(seq).to(dev), kv_slot=torch.from_numpy(kv).to(dev), tables=torch.from_numpy(bt).to(dev),
+                   row_req=torch.from_numpy(np.repeat(np.arange(B, dtype=np.int32), np.asarray(counts, dtype=np.int64))).to(dev),
+                   pos=torch.from_numpy(row_pos).to(dev),
                    page_size=int(page_size), max_pos=max(int(s) + int(c) for s, c in zip(starts, counts)), max_page=int(bt.max()),
                    max_slot=int(max(slots)), _tiles={})
 
@@ -168,8 +174,8 @@ def qk_norm_append(proj: torch.Tensor, cols: Tuple[int, int, int], H: int, G: in
     return q
 
 
-def attn_tile_rows(dtype: torch.dtype, H: int, G: int, D: int, Dv: int) -> int:
-    tq = int(N.layers().jl_attn_tile_rows(_code(dtype), H, G, D, Dv))
+def attn_tile_rows(dtype: torch.dtype, H: int, G: int, D: int, Dv: int, k_ld: int = 0, v_ld: int = 0) -> int:
+    tq = int(N.layers().jl_attn_tile_rows(_code(dtype), H, G, D, Dv, k_ld, v_ld))
     if tq <= 0:
         raise ValueError(f"attention sizes heads={H} kv_heads={G} dim={D} vdim={Dv} exceed the kernel's tile")
     return tq
@@ -177,13 +183,20 @@ def attn_tile_rows(dtype: torch.dtype, H: int, G: int, D: int, Dv: int) -> int:
 
 def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Tensor, v_cache: torch.Tensor, batch: RaggedBatch,
                 H: int, G: int, D: int, Dv: int, scale: float, window: int, keep_first: int, rel: Optional[torch.Tensor],
-                lut: Optional[torch.Tensor], talk: Optional[torch.Tensor]) -> torch.Tensor:
-    """q [N, H*D]; gate a [N, H*Dv] view (column range of the projection output, row stride free) or None.  Returns [N, H*Dv]."""
+                lut: Optional[torch.Tensor], talk: Optional[torch.Tensor], value_heads: int = 0, float_out: bool = False) -> torch.Tensor:
+    """q [N, H*D]; gate a [N, H*Dv] view (column range of the projection output, row stride free) or None.  Returns [N, H*Dv].
+    The pools may be column ranges of wider rows (``v_cache`` may be a view into ``k_cache``).  ``value_heads`` (0: G) < G: key head
+    c reads value head c % value_heads — several score maps over the same values.  ``float_out``: float outputs from bfloat16
+    inputs (for what is subtracted or normalised next)."""
     _dev(q)
     dt = q.dtype
     n = q.shape[0]
+    Gv = value_heads or G
     _need(q.is_contiguous() and q.shape[1] == H * D and n == batch.N, "attn_window: q [N, H*D] of the batch")
-    _need(k_cache.dtype == dt and v_cache.dtype == dt and k_cache.shape[-1] == G * D and v_cache.shape[-1] == G * Dv, "attn_window: pool dtype / widths")
+    _need(G % Gv == 0 and k_cache.dtype == dt and v_cache.dtype == dt and k_cache.dim() == 2 and v_cache.dim() == 2 and k_cache.shape[1] == G * D and
+          v_cache.shape[1] == Gv * Dv and k_cache.stride(1) == 1 and v_cache.stride(1) == 1 and k_cache.shape[0] == v_cache.shape[0],
+          "attn_window: pool dtype / widths")
+    k_ld, v_ld = k_cache.stride(0), v_cache.stride(0)
     pool_tokens = k_cache.shape[0]
     _need(pool_tokens % batch.page_size == 0 and batch.max_page < pool_tokens // batch.page_size, "attn_window: a page lies outside the pool")
     if gate is not None:
@@ -193,9 +206,9 @@ def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Te
             _need(t.dtype == torch.float32 and t.is_contiguous() and (shape is None or tuple(t.shape) == shape), "attn_window: float tables")
     if rel is not None:                                  # rel [rows, H] with lut [positions] -> row, or rel [positions, H] by distance itself
         _need(rel.shape[1] == H and (lut is None or lut.dtype == torch.int32), "attn_window: rel [rows, H] (+ int32 lut)")
-    tq = attn_tile_rows(dt, H, G, D, Dv)
+    tq = attn_tile_rows(dt, H, G, D, Dv, k_ld, v_ld)
     tiles = batch.tiles(tq)
-    out = torch.empty((n, H * Dv), dtype=dt, device=q.device)
+    out = torch.empty((n, H * Dv), dtype=torch.float32 if float_out else dt, device=q.device)
     # few tiles with many keys (decoding): share each tile's keys out over workgroups until the chip is full
     splits, scratch = 1, None
     if tq == 32 and tiles.shape[0] < ATTN_SPLIT_BELOW_TILES:
@@ -211,7 +224,8 @@ def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Te
                    lut_len=(lut.numel() if lut is not None else rel.shape[0]) if rel is not None else 0, page_size=batch.page_size, H=H, G=G, D=D, Dv=Dv, window=int(window),
                    keep_first=int(keep_first), TQ=tq, dtype=_code(dt), scale=float(scale), splits=splits, n_rows=n,
                    scratch=scratch.data_ptr() if scratch is not None else None,
-                   q_pack=q_pack.data_ptr() if q_pack is not None else None)
+                   q_pack=q_pack.data_ptr() if q_pack is not None else None, k_ld=k_ld, v_ld=v_ld, Gv=Gv,
+                   out_dtype=N.JL_OUT_F32 if float_out and dt != torch.float32 else N.JL_OUT_SAME)
     N.check_layers(N.layers().jl_attn_window(C.byref(a), _stream(q.device)), "jl_attn_window")
     return out
 
@@ -284,3 +298,126 @@ def moe_experts(h: torch.Tensor, router_logits: torch.Tensor, correction: Option
     N.check_layers(L.jl_moe_gemm(_ptr(act), _ptr(w_down), _code(dt), 1, ff, W, top, _ptr(perm), _ptr(offsets), _ptr(tile_e), _ptr(tile_r), max_tiles,
                                  _ptr(wts), _ptr(y), st), "jl_moe_gemm(down)")
     return y
+
+
+def norm_add(x: torch.Tensor, y: torch.Tensor, g: torch.Tensor, eps: float, out_dtype: Optional[torch.dtype]) -> Optional[torch.Tensor]:
+    """x (float [N, W], in place) += rms_norm(y) * g, g a single float (a norm on a sublayer's OUTPUT).  Returns x in
+    ``out_dtype`` (None: the update only)."""
+    _dev(x)
+    n, W = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and tuple(y.shape) == (n, W), "norm_add: x float [N, W], y [N, W]")
+    _need(g.dtype == torch.float32 and g.numel() == 1, "norm_add: the weight is one float")
+    out = torch.empty((n, W), dtype=out_dtype, device=x.device) if out_dtype is not None else None
+    N.check_layers(N.layers().jl_norm_add(_ptr(x), _ptr(y), _code(y.dtype), _ptr(g), float(eps), _ptr(out), _code(out_dtype or torch.float32), n, W,
+                                         _stream(x.device)), "jl_norm_add")
+    return out
+
+
+def polynorm(z: torch.Tensor, coef: torch.Tensor, eps: float) -> torch.Tensor:
+    """c0 n(z) + c1 n(z^2) + c2 n(z^3) + c3 with n(u) = u / rms(u) over a row; z [N, F], coef four floats."""
+    _dev(z)
+    _need(z.dim() == 2 and z.is_contiguous() and coef.dtype == torch.float32 and coef.numel() == 4 and coef.is_contiguous(), "polynorm: z [N, F], coef float [4]")
+    out = torch.empty_like(z)
+    N.check_layers(N.layers().jl_polynorm(_ptr(z), _code(z.dtype), z.shape[0], z.shape[1], _ptr(coef), float(eps), _ptr(out), _stream(z.device)),
+                   "jl_polynorm")
+    return out
+
+
+def causal_conv(x: torch.Tensor, w: torch.Tensor, batch: RaggedBatch, tail: Optional[torch.Tensor]) -> torch.Tensor:
+    """x + (causal depthwise convolution of x over time, per request), from the float residual x [N, W] with w [W, taps]; ``tail``
+    float [slots, taps - 1, W] carries every request's last inputs from step to step (updated here).  Returns [N, W] of w's dtype."""
+    _dev(x)
+    n, W = x.shape
+    taps = w.shape[1]
+    _need(x.dtype == torch.float32 and x.is_contiguous() and n == batch.N and w.is_contiguous() and w.shape[0] == W, "causal_conv: x float [N, W], w [W, taps]")
+    if taps > 1:
+        _need(tail is not None and tail.dtype == torch.float32 and tail.is_contiguous() and tuple(tail.shape[1:]) == (taps - 1, W) and
+              batch.max_slot < tail.shape[0], "causal_conv: tail float [slots, taps - 1, W] with the batch's slots")
+    out = torch.empty((n, W), dtype=w.dtype, device=x.device)
+    L, st = N.layers(), _stream(x.device)
+    N.check_layers(L.jl_causal_conv(_ptr(x), _ptr(w), _code(w.dtype), _ptr(batch.row_req), _ptr(batch.seq), _ptr(tail), n, W, taps, _ptr(out), st),
+                   "jl_causal_conv")
+    if taps > 1:
+        N.check_layers(L.jl_causal_conv_carry(_ptr(x), _ptr(batch.seq), batch.B, _ptr(tail), W, taps, st), "jl_causal_conv_carry")
+    return out
+
+
+def head_norm_append(proj: torch.Tensor, cols: Tuple[int, int, int], H: int, G: int, M: int, D: int, Dv: int, wq: torch.Tensor, wk: torch.Tensor,
+                     eps: float, t_coef: float, t_every: int, batch: RaggedBatch, k_cache: torch.Tensor, v_cache: torch.Tensor) -> torch.Tensor:
+    """Per-head (and per score map) RMS norm of q and k over D, query temperature by position, keys / values appended to the
+    pools.  Returns q [N, M*H*D] map-major; the key pool rows are [M, G, D] map-major."""
+    _dev(proj)
+    n, ld = proj.shape
+    dt = proj.dtype
+    _need(proj.is_contiguous() and n == batch.N, "head_norm_append: proj [N, ld] of the batch")
+    _need(wq.numel() == D and wk.numel() == D and wq.dtype == dt and wk.dtype == dt, "head_norm_append: norm weights over one head")
+    _need(k_cache.dtype == dt and v_cache.dtype == dt and k_cache.is_contiguous() and v_cache.is_contiguous() and
+          k_cache.shape[-1] == M * G * D and v_cache.shape[-1] == G * Dv and k_cache.shape[0] == v_cache.shape[0], "head_norm_append: pools [tokens, M*G*D] / [tokens, G*Dv]")
+    q = torch.empty((n, M * H * D), dtype=dt, device=proj.device)
+    N.check_layers(N.layers().jl_head_norm_append(_ptr(proj), _code(dt), n, ld, cols[0], cols[1], cols[2], H, G, M, D, Dv, _ptr(wq), _ptr(wk), float(eps),
+                                                 float(t_coef), int(t_every), _ptr(batch.pos), _ptr(q), _ptr(k_cache), _ptr(v_cache),
+                                                 _ptr(batch.kv_slot), _stream(proj.device)), "jl_head_norm_append")
+    return q
+
+
+def diff_combine(a: torch.Tensor, H: int, Dv: int, lam: float, eps: float, out_scale: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """a float [N, 2*H*Dv] (two score maps' outputs, map-major) -> rms_norm_per_head(a[0] - lam * a[1]) * out_scale, [N, H*Dv]."""
+    _dev(a)
+    n = a.shape[0]
+    _need(a.dtype == torch.float32 and a.is_contiguous() and a.shape[1] == 2 * H * Dv, "diff_combine: a float [N, 2*H*Dv]")
+    out = torch.empty((n, H * Dv), dtype=out_dtype, device=a.device)
+    N.check_layers(N.layers().jl_diff_combine(_ptr(a), n, H, Dv, float(lam), float(eps), float(out_scale), _ptr(out), _code(out_dtype),
+                                             _stream(a.device)), "jl_diff_combine")
+    return out
+
+
+def _angle_tables(rot_dims: int, cos, sin, batch: RaggedBatch, what: str) -> int:
+    if not rot_dims:
+        return 0
+    _need(cos is not None and cos.dtype == torch.float32 and cos.is_contiguous() and cos.shape == sin.shape and cos.shape[1] == rot_dims // 2,
+          f"{what}: cos / sin [positions, rot_dims / 2] float")
+    _need(batch.max_pos <= cos.shape[0], f"{what}: the angle tables are shorter than the batch's positions")
+    return cos.shape[0]
+
+
+def latent_prep(proj: torch.Tensor, q_col: int, Rq: int, kv_col: int, R: int, rd: int, rot_dims: int, wq: torch.Tensor, wkv: torch.Tensor,
+                eps: float, batch: RaggedBatch, cos, sin, pool: torch.Tensor) -> torch.Tensor:
+    """Normalised query latent [N, Rq]; the pool row of every token becomes [normalised key/value latent | rotated shared key]."""
+    _dev(proj)
+    n, ld = proj.shape
+    dt = proj.dtype
+    _need(proj.is_contiguous() and n == batch.N and wq.numel() == Rq and wkv.numel() == R and wq.dtype == dt and wkv.dtype == dt,
+          "latent_prep: proj [N, ld] of the batch, norm weights over the latents")
+    _need(pool.dtype == dt and pool.is_contiguous() and pool.shape[-1] == R + rd, "latent_prep: pool [tokens, R + rd]")
+    tl = _angle_tables(rot_dims, cos, sin, batch, "latent_prep")
+    cq = torch.empty((n, Rq), dtype=dt, device=proj.device)
+    N.check_layers(N.layers().jl_latent_prep(_ptr(proj), _code(dt), n, ld, q_col, Rq, kv_col, R, rd, rot_dims, _ptr(wq), _ptr(wkv), float(eps),
+                                            _ptr(batch.pos), _ptr(cos), _ptr(sin), tl, _ptr(cq), _ptr(pool), _ptr(batch.kv_slot),
+                                            _stream(proj.device)), "jl_latent_prep")
+    return cq
+
+
+def latent_q_pack(qa: torch.Tensor, q: torch.Tensor, H: int, D: int, R: int, rd: int, rot_dims: int, batch: RaggedBatch, cos, sin) -> torch.Tensor:
+    """qa [H, N, R] (queries times the key up-projection), q [N, H*(D + rd)] -> [N, H*(R + rd)] with the rotary part rotated."""
+    _dev(q)
+    n = q.shape[0]
+    _need(q.is_contiguous() and qa.is_contiguous() and tuple(qa.shape) == (H, n, R) and q.shape[1] == H * (D + rd) and qa.dtype == q.dtype and n == batch.N,
+          "latent_q_pack: qa [H, N, R], q [N, H*(D + rd)]")
+    tl = _angle_tables(rot_dims, cos, sin, batch, "latent_q_pack")
+    out = torch.empty((n, H * (R + rd)), dtype=q.dtype, device=q.device)
+    N.check_layers(N.layers().jl_latent_q_pack(_ptr(qa), _ptr(q), _code(q.dtype), n, H, D, R, rd, rot_dims, _ptr(batch.pos), _ptr(cos), _ptr(sin), tl,
+                                              _ptr(out), _stream(q.device)), "jl_latent_q_pack")
+    return out
+
+
+def heads_gate(ov: torch.Tensor, gate: Optional[torch.Tensor]) -> torch.Tensor:
+    """ov [H, N, Dv] -> [N, H*Dv], times sigmoid(gate) (a [N, H*Dv] view, row stride free)."""
+    _dev(ov)
+    H, n, Dv = ov.shape
+    _need(ov.is_contiguous(), "heads_gate: ov [H, N, Dv] contiguous")
+    if gate is not None:
+        _need(gate.shape == (n, H * Dv) and gate.stride(1) == 1 and gate.dtype == ov.dtype, "heads_gate: gate [N, H*Dv]")
+    out = torch.empty((n, H * Dv), dtype=ov.dtype, device=ov.device)
+    N.check_layers(N.layers().jl_heads_gate(_ptr(ov), _ptr(gate), gate.stride(0) if gate is not None else 0, _code(ov.dtype), n, H, Dv, _ptr(out),
+                                           _stream(ov.device)), "jl_heads_gate")
+    return out

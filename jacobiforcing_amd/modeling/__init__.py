@@ -13,6 +13,7 @@ from pathlib import Path
 MODEL_REGISTRY = {
     "Qwen2ForCausalLM": ("jacobiforcing_amd.modeling.qwen2", "Qwen2Config", "padded"),
     "Lokizen": ("jacobiforcing_amd.modeling.lokizen", "LokizenConfig", "ragged"),
+    "Vumalix": ("jacobiforcing_amd.modeling.vumalix", "VumalixConfig", "ragged"),
 }
 
 
