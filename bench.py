@@ -730,8 +730,8 @@ def main():
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=96)
-    ap.add_argument("--design", default="", help="'lokizen': instead of the default workload, prefill / decode throughput of the ragged Lokizen "
-                    "family at real-layer sizes beside Qwen2 at equal size, and each layer kernel against its roofline (one JSON line)")
+    ap.add_argument("--design", default="", help="'lokizen' / 'vumalix': instead of the default workload, prefill / decode throughput of that ragged "
+                    "family at real-layer sizes beside the closest existing model at equal size, and each layer kernel against its roofline (one JSON line)")
     ap.add_argument("--design-sizes", default="small,medium")
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--prompts-per-gpu", type=int, default=64, help="weak scaling: prompts decoded by every rank")
@@ -755,12 +755,12 @@ def main():
     if args.gpus < 1:
         raise SystemExit("--gpus must be >= 1")
     if args.design:
-        if args.design.lower() != "lokizen":
-            raise SystemExit(f"--design {args.design}: only 'lokizen' has a comparison section")
+        if args.design.lower() not in ("lokizen", "vumalix"):
+            raise SystemExit(f"--design {args.design}: only 'lokizen' and 'vumalix' have a comparison section")
         if not torch.cuda.is_available():
             raise SystemExit("bench.py needs an MI355X: the layer kernels have no CPU path")
         from jacobiforcing_amd.drivers import ragged_bench
-        print(json.dumps(ragged_bench.run(tuple(args.design_sizes.split(",")))), flush=True)
+        print(json.dumps(ragged_bench.run(tuple(args.design_sizes.split(",")), design=args.design)), flush=True)
         return
     if args.gpus > 1 and "WORLD_SIZE" not in os.environ:
         sys.exit(spawn_ranks(args.gpus, sys.argv[1:]))          # plain command: start the N ranks, relay their exit code

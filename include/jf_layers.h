@@ -74,6 +74,16 @@ JL_API int jl_attn_window(const jl_attn_args *a, void *stream);
  * they do not fit */
 JL_API int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv, int64_t k_ld, int64_t v_ld);
 
+/* The same attention for ONE key/value head shared by all H query heads whose values are the first Dv columns of the key rows (the
+ * pool of latent attention), on the matrix cores in one sweep: bfloat16, G = 1, D % 8 == 0 up to 640, Dv in {128, 256, 384, 512} <= D,
+ * k_ld % 4 == 0; no bias, head mixing or gate.  Of jl_attn_args it reads q, k_cache, k_ld, out, block_tables, bt_stride, tiles, n_tiles,
+ * page_size, H, G, D, Dv, window, scale, dtype and TQ, which must be what jl_attn_shared_kv_tile_rows returns (0: sizes not taken). */
+JL_API int jl_attn_shared_kv(const jl_attn_args *a, void *stream);
+JL_API int jl_attn_shared_kv_tile_rows(int dtype, int32_t H, int32_t D, int32_t Dv, int64_t k_ld);
+/* splits in 2 .. 64: the keys of every tile are shared out over that many workgroups and joined by a second launch; `scratch` then
+ * holds this many floats */
+JL_API int64_t jl_attn_shared_kv_scratch_floats(int32_t n_tiles, int32_t H, int32_t Dv, int32_t splits);
+
 /* Sublayer-output norm + residual update: x[n] += y[n] / sqrt(mean(y[n]^2) + eps) * g[0] (x float in place, y of y_dtype, g one
  * float); when `out` is given, out[n] = x[n] in `out_dtype` (what the next sublayer's product reads). */
 JL_API int jl_norm_add(float *x, const void *y, int y_dtype, const float *g, float eps, void *out, int out_dtype, int64_t N, int32_t W,
@@ -87,10 +97,11 @@ JL_API int jl_polynorm(const void *z, int dtype, int64_t N, int32_t F, const flo
  *   out[t, c] = x[t, c] + sum_{j < taps} w[c, j] * x[t - taps + 1 + j, c]        (zeros before the sequence's start)
  * x float [N, W]; w [W, taps] and out [N, W] of `dtype`; row_req [N] int32 the request of every row; seq [B, 4] as above;
  * tail float [slots, taps - 1, W]: the inputs at positions pos0 - taps + 1 .. pos0 - 1 of the slot's request (entries before
- * position 0 are never read, so a slot's old content does not matter to a new request).  jl_causal_conv reads the tail;
- * jl_causal_conv_carry, enqueued after it, moves it to the end of the step's rows.  taps <= JL_CONV_MAX_TAPS. */
+ * position 0 are never read, so a slot's old content does not matter to a new request).  jl_causal_conv reads the tail and, for a
+ * request with ONE row in the step, moves it on; jl_causal_conv_carry, enqueued after it, does that for the requests with more rows
+ * (not needed when no request has more than one).  taps <= JL_CONV_MAX_TAPS. */
 #define JL_CONV_MAX_TAPS 16
-JL_API int jl_causal_conv(const float *x, const void *w, int dtype, const int32_t *row_req, const int32_t *seq, const float *tail,
+JL_API int jl_causal_conv(const float *x, const void *w, int dtype, const int32_t *row_req, const int32_t *seq, float *tail,
                           int64_t N, int32_t W, int32_t taps, void *out, void *stream);
 JL_API int jl_causal_conv_carry(const float *x, const int32_t *seq, int32_t B, float *tail, int32_t W, int32_t taps, void *stream);
 
@@ -99,16 +110,17 @@ JL_API int jl_causal_conv_carry(const float *x, const int32_t *seq, int32_t B, f
  * its own and multiplied by wq / wk [D]; the query is further multiplied by 1 + t_coef * ln(floor((p + 1) / t_every) + 1), p = pos[n]
  * (t_coef 0: no temperature).  Queries and keys are written MAP-major — q_out [N, M, H, D], k_cache[slot[n]] = [M, G, D] — so that
  * query row m*H + h reads key row (m*H + h) / (H/G) = m*G + h/(H/G) and value head (m*G + g) % G: one attention launch with M*H query
- * heads, M*G key heads and G value heads computes all maps.  v goes to v_cache[slot[n]] as it is. */
+ * heads, M*G key heads and G value heads computes all maps.  With maps_apart != 0 the queries are written [M, N, H, D] instead: one
+ * launch per map, each over its own G*D columns of the key rows.  v goes to v_cache[slot[n]] as it is. */
 JL_API int jl_head_norm_append(const void *proj, int dtype, int64_t N, int64_t ld, int32_t q_col, int32_t k_col, int32_t v_col, int32_t H,
                                int32_t G, int32_t M, int32_t D, int32_t Dv, const void *wq, const void *wk, float eps, float t_coef,
-                               int32_t t_every, const int32_t *pos, void *q_out, void *k_cache, void *v_cache, const int64_t *slot,
-                               void *stream);
+                               int32_t t_every, const int32_t *pos, void *q_out, int32_t maps_apart, void *k_cache, void *v_cache,
+                               const int64_t *slot, void *stream);
 
-/* Differential combination of two score maps' outputs: a float [N, 2, H, Dv] (map-major, as the launch above produces);
- * o = a[0] - lambda * a[1];  out[n, h] = o / sqrt(mean(o^2) + eps) * out_scale over the head's Dv values; out [N, H*Dv] of `dtype`. */
-JL_API int jl_diff_combine(const float *a, int64_t N, int32_t H, int32_t Dv, float lambda, float eps, float out_scale, void *out,
-                           int dtype, void *stream);
+/* Differential combination of two score maps' outputs a1, a2 (float, rows of H*Dv values `ld` floats apart):
+ * o = a1 - lambda * a2;  out[n, h] = o / sqrt(mean(o^2) + eps) * out_scale over the head's Dv values; out [N, H*Dv] of `dtype`. */
+JL_API int jl_diff_combine(const float *a1, const float *a2, int64_t ld, int64_t N, int32_t H, int32_t Dv, float lambda, float eps,
+                           float out_scale, void *out, int dtype, void *stream);
 
 /* Latent attention, input side.  proj [N, ld] holds the query latent (Rq columns at q_col) and the key/value latent (R columns at
  * kv_col) followed by rd rotary key dimensions shared by all heads.

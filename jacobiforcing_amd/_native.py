@@ -230,7 +230,6 @@ def raise_state_error(code: int, what: str, aux: int = 0):
 
 
 # ---- libjf_layers.so (include/jf_layers.h): layer kernels of the models whose forward is not stock PyTorch ----------------------------
-LAYERS_LIB_PATH = _PKG / "lib" / "libjf_layers.so"
 JL_F32, JL_BF16 = 0, 1
 JL_OUT_SAME, JL_OUT_F32 = 0, 2
 
@@ -254,13 +253,16 @@ _LAYER_SIGNATURES = {
     "jl_attn_window": (C.c_int, [C.POINTER(AttnArgs), _vp]),
     "jl_attn_scratch_floats": (_i64, [_i32, _i32, _i32, _i32, _i32]),
     "jl_attn_tile_rows": (C.c_int, [C.c_int, _i32, _i32, _i32, _i32, _i64, _i64]),
+    "jl_attn_shared_kv": (C.c_int, [C.POINTER(AttnArgs), _vp]),
+    "jl_attn_shared_kv_tile_rows": (C.c_int, [C.c_int, _i32, _i32, _i32, _i64]),
+    "jl_attn_shared_kv_scratch_floats": (_i64, [_i32, _i32, _i32, _i32]),
     "jl_norm_add": (C.c_int, [_vp, _vp, C.c_int, _vp, _f32, _vp, C.c_int, _i64, _i32, _vp]),
     "jl_polynorm": (C.c_int, [_vp, C.c_int, _i64, _i32, _vp, _f32, _vp, _vp]),
     "jl_causal_conv": (C.c_int, [_vp, _vp, C.c_int, _vp, _vp, _vp, _i64, _i32, _i32, _vp, _vp]),
     "jl_causal_conv_carry": (C.c_int, [_vp, _vp, _i32, _vp, _i32, _i32, _vp]),
     "jl_head_norm_append": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _f32, _i32,
-                                      _vp, _vp, _vp, _vp, _vp, _vp]),
-    "jl_diff_combine": (C.c_int, [_vp, _i64, _i32, _i32, _f32, _f32, _f32, _vp, C.c_int, _vp]),
+                                      _vp, _vp, _i32, _vp, _vp, _vp, _vp]),
+    "jl_diff_combine": (C.c_int, [_vp, _vp, _i64, _i64, _i32, _i32, _f32, _f32, _f32, _vp, C.c_int, _vp]),
     "jl_latent_prep": (C.c_int, [_vp, C.c_int, _i64, _i64, _i32, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _f32, _vp, _vp, _vp, _i64, _vp, _vp,
                                  _vp, _vp]),
     "jl_latent_q_pack": (C.c_int, [_vp, _vp, C.c_int, _i64, _i32, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _i64, _vp, _vp]),
@@ -274,21 +276,28 @@ _LAYER_SIGNATURES = {
     "jl_moe_gemm": (C.c_int, [_vp, _vp, C.c_int, _i32, _i32, _i32, _i32, _vp, _vp, _vp, _vp, _i32, _vp, _vp, _vp]),
 }
 LAYER_SYMBOLS = tuple(_LAYER_SIGNATURES)
-_LAYERS = None
+# which library a symbol lives in (jacobiforcing_amd/_build.py: LAYER_GROUPS); both carry their own jl_version / jl_last_error
+_SEQ_SYMBOLS = ("jl_retention", "jl_retention_join", "jl_moe_route", "jl_moe_group", "jl_moe_tile_rows", "jl_moe_gemm")
 
 
-def layers():
-    """The layer-kernel library.  Loads what is built; compiles it (hipcc, about a minute) only when there is none — a fresh
-    checkout's first call.  There is no CPU or eager fallback for these kernels either."""
-    global _LAYERS
-    if _LAYERS is None:
-        p = Path(os.environ.get("JF_LAYERS_LIB", LAYERS_LIB_PATH))
+class _LayerLibs:
+    """The layer-kernel libraries behind one attribute namespace.  A library is loaded at the first use of one of its symbols:
+    what is built is loaded; when there is none it is compiled (hipcc, about a minute for the attention kernels) — a fresh
+    checkout's first call compiles only the library its model launches.  There is no CPU or eager fallback for these kernels."""
+
+    def __init__(self):
+        self._libs = {}
+        self._last = None
+
+    def _load(self, group: str):
+        from . import _build
+        env = {"layers": "JF_LAYERS_LIB", "layers_seq": "JF_LAYERS_SEQ_LIB"}[group]
+        p = Path(os.environ.get(env, _build.layer_lib(group)))
         if not p.exists():
-            if "JF_LAYERS_LIB" in os.environ:
+            if env in os.environ:
                 raise NativeLibraryError(f"{p} not found")
-            from . import _build
             try:
-                _build.build_layers()
+                _build.build_layers(groups=[group])
             except Exception as e:
                 raise NativeLibraryError(f"cannot build {p}: {e}") from e
         try:
@@ -296,12 +305,35 @@ def layers():
         except OSError as e:
             raise NativeLibraryError(f"cannot load {p}: {e}") from e
         for name, (res, args) in _LAYER_SIGNATURES.items():
+            if (name in _SEQ_SYMBOLS) != (group == "layers_seq") and name not in ("jl_version", "jl_last_error"):
+                continue
             try:
                 fn = getattr(lib_, name)
             except AttributeError as e:
                 raise NativeLibraryError(f"{p} does not export {name}") from e
             fn.restype, fn.argtypes = res, args
-        _LAYERS = lib_
+        self._libs[group] = lib_
+        return lib_
+
+    def __getattr__(self, name: str):
+        if name.startswith("_"):
+            raise AttributeError(name)
+        if name == "jl_last_error":                  # the message of the library that was called last
+            return (self._last or self._libs.get("layers") or self._load("layers")).jl_last_error
+        group = "layers_seq" if name in _SEQ_SYMBOLS else "layers"
+        self._last = self._libs.get(group) or self._load(group)
+        return getattr(self._last, name)
+
+
+_LAYERS = None
+
+
+def layers():
+    global _LAYERS
+    if _LAYERS is None:
+        _LAYERS = _LayerLibs()
+    if "layers" not in _LAYERS._libs:               # the attention / norm library is what every ragged family needs: load (or build) it now
+        _LAYERS._load("layers")
     return _LAYERS
 
 

@@ -611,7 +611,7 @@ __global__ __launch_bounds__(256) void attn_join_kernel(const float *__restrict_
 
 static bool am_fits(int dtype, int H, int G, int D, int Dv) {
     static const bool off = getenv("JL_ATTN_NO_MFMA") != nullptr;          // A/B switch for measurements
-    return !off && dtype == JL_BF16 && H <= 16 && D % 8 == 0 && D <= 256 && Dv <= 128 && Dv % 4 == 0 &&
+    return !off && dtype == JL_BF16 && H <= 16 && D % 8 == 0 && D <= 640 && Dv <= 128 && Dv % 4 == 0 &&
            am_lds_bytes(H, G, D, Dv) <= (size_t)ATT_LDS_BUDGET + 8 * 1024;
 }
 

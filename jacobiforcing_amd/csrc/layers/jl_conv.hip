@@ -3,14 +3,16 @@
 #include "jl_common.h"
 
 // one workgroup per row; a thread per channel.  Input t - taps + 1 + j of the request comes from the step's own rows when it is
-// one of them, from the slot's tail when it lies before the step, and is zero before the sequence's start.
+// one of them, from the slot's tail when it lies before the step, and is zero before the sequence's start.  A request with ONE row in
+// the step (decoding) also moves its tail here — its only reader is this thread, which has read what it needs; requests with more
+// rows leave that to causal_conv_carry_kernel, after every row has read.
 template <typename T>
 __global__ __launch_bounds__(256) void causal_conv_kernel(const float *__restrict__ x, const T *__restrict__ w, const int32_t *__restrict__ row_req,
-                                                           const int32_t *__restrict__ seq, const float *__restrict__ tail, int W, int taps,
+                                                           const int32_t *__restrict__ seq, float *tail, int W, int taps,
                                                            T *__restrict__ out) {
     const int64_t n = blockIdx.x;
     const int32_t *rec = seq + 4 * (int64_t)row_req[n];
-    const int row0 = rec[0], pos0 = rec[2], slot = rec[3];
+    const int row0 = rec[0], count = rec[1], pos0 = rec[2], slot = rec[3];
     const int t = (int)(n - row0), keep = taps - 1;
     for (int c = threadIdx.x; c < W; c += 256) {
         float acc = x[n * W + c];
@@ -22,10 +24,15 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const float *__restric
             acc += ld_f(w + (int64_t)c * taps + j) * v;
         }
         st_f(out + n * W + c, acc);
+        if (count == 1 && keep > 0) {                           // the tail moves one place on: entry j was read before entry j - 1 is written
+            float *tl = tail + (int64_t)slot * keep * W + c;
+            for (int j = 1; j < keep; ++j) tl[(int64_t)(j - 1) * W] = tl[(int64_t)j * W];
+            tl[(int64_t)(keep - 1) * W] = x[n * W + c];
+        }
     }
 }
 
-extern "C" int jl_causal_conv(const float *x, const void *w, int dtype, const int32_t *row_req, const int32_t *seq, const float *tail,
+extern "C" int jl_causal_conv(const float *x, const void *w, int dtype, const int32_t *row_req, const int32_t *seq, float *tail,
                               int64_t N, int32_t W, int32_t taps, void *out, void *stream) {
     if (N <= 0) return JL_OK;
     if (!x || !w || !row_req || !seq || !out || W <= 0 || taps < 1 || taps > JL_CONV_MAX_TAPS || (taps > 1 && !tail))
@@ -42,7 +49,7 @@ __global__ __launch_bounds__(256) void causal_conv_carry_kernel(const float *__r
     const int32_t *rec = seq + 4 * (int64_t)blockIdx.y;
     const int row0 = rec[0], count = rec[1], pos0 = rec[2], slot = rec[3], keep = taps - 1;
     const int c = blockIdx.x * 256 + threadIdx.x;
-    if (c >= W || count <= 0) return;
+    if (c >= W || count <= 1) return;                       // a single row has moved its tail in causal_conv_kernel
     float v[JL_CONV_MAX_TAPS];
 #pragma unroll
     for (int s = 0; s < JL_CONV_MAX_TAPS - 1; ++s) {

@@ -7,7 +7,8 @@ template <typename T>
 __global__ __launch_bounds__(256) void head_norm_append_kernel(const T *__restrict__ proj, int64_t ld, int q_col, int k_col, int v_col, int H, int G,
                                                                 int M, int D, int GDv, const T *__restrict__ wq, const T *__restrict__ wk, float eps,
                                                                 float t_coef, int t_every, const int32_t *__restrict__ pos, T *__restrict__ q_out,
-                                                                T *__restrict__ k_cache, T *__restrict__ v_cache, const int64_t *__restrict__ slot) {
+                                                                int64_t q_map_stride, T *__restrict__ k_cache, T *__restrict__ v_cache,
+                                                                const int64_t *__restrict__ slot) {
     const int64_t n = blockIdx.x;
     const T *row = proj + n * ld;
     const int wave = threadIdx.x >> 6, lane = threadIdx.x & 63;
@@ -25,7 +26,9 @@ __global__ __launch_bounds__(256) void head_norm_append_kernel(const T *__restri
         ss = wave_sum_f32(ss);
         const float r = 1.0f / sqrtf(ss / (float)D + eps);
         if (is_q) {
-            T *dst = q_out + n * ((int64_t)nq * D) + ((int64_t)map * H + head) * D;
+            // q_map_stride 0: [N, M, H, D]; else [M, N, H, D] with the maps q_map_stride elements apart
+            T *dst = q_map_stride ? q_out + map * q_map_stride + n * ((int64_t)H * D) + (int64_t)head * D
+                                  : q_out + n * ((int64_t)nq * D) + ((int64_t)map * H + head) * D;
             for (int d = lane; d < D; d += 64) st_f(dst + d, ld_f(src + d) * r * ld_f(wq + d) * temp);
         } else if (sl >= 0) {
             T *dst = k_cache + sl * ((int64_t)nk * D) + ((int64_t)map * G + head) * D;
@@ -38,8 +41,8 @@ __global__ __launch_bounds__(256) void head_norm_append_kernel(const T *__restri
 
 extern "C" int jl_head_norm_append(const void *proj, int dtype, int64_t N, int64_t ld, int32_t q_col, int32_t k_col, int32_t v_col, int32_t H,
                                    int32_t G, int32_t M, int32_t D, int32_t Dv, const void *wq, const void *wk, float eps, float t_coef,
-                                   int32_t t_every, const int32_t *pos, void *q_out, void *k_cache, void *v_cache, const int64_t *slot,
-                                   void *stream) {
+                                   int32_t t_every, const int32_t *pos, void *q_out, int32_t maps_apart, void *k_cache, void *v_cache,
+                                   const int64_t *slot, void *stream) {
     if (N <= 0) return JL_OK;
     if (!proj || !wq || !wk || !q_out || !k_cache || !v_cache || !slot) return jl_fail(JL_E_INVALID, "jl_head_norm_append: null pointer");
     if (H <= 0 || G <= 0 || M <= 0 || D <= 0 || Dv <= 0 || q_col + (int64_t)H * M * D > ld || k_col + (int64_t)G * M * D > ld || v_col + (int64_t)G * Dv > ld)
@@ -47,20 +50,20 @@ extern "C" int jl_head_norm_append(const void *proj, int dtype, int64_t N, int64
     if (t_coef != 0.f && (!pos || t_every <= 0)) return jl_fail(JL_E_INVALID, "jl_head_norm_append: a query temperature needs positions and a period >= 1");
     JL_DISPATCH(dtype, head_norm_append_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(
                            (const T *)proj, ld, q_col, k_col, v_col, H, G, M, D, G * Dv, (const T *)wq, (const T *)wk, eps, t_coef, t_every, pos,
-                           (T *)q_out, (T *)k_cache, (T *)v_cache, slot));
+                           (T *)q_out, maps_apart ? N * (int64_t)H * D : 0, (T *)k_cache, (T *)v_cache, slot));
     return jl_check_launch("head_norm_append_kernel");
 }
 
 // o = a[map 0] - lambda * a[map 1], unit RMS per head, times out_scale.  A wavefront per (token, head).
 template <typename T>
-__global__ __launch_bounds__(256) void diff_combine_kernel(const float *__restrict__ a, int64_t N, int H, int Dv, float lambda, float eps,
-                                                            float out_scale, T *__restrict__ out) {
+__global__ __launch_bounds__(256) void diff_combine_kernel(const float *__restrict__ m1, const float *__restrict__ m2, int64_t ld, int64_t N, int H,
+                                                            int Dv, float lambda, float eps, float out_scale, T *__restrict__ out) {
     const int64_t vec = (int64_t)blockIdx.x * 4 + (threadIdx.x >> 6);
     if (vec >= N * H) return;
     const int lane = threadIdx.x & 63;
     const int64_t n = vec / H;
     const int h = (int)(vec - n * H);
-    const float *a1 = a + (n * 2 * H + h) * (int64_t)Dv, *a2 = a1 + (int64_t)H * Dv;
+    const float *a1 = m1 + n * ld + (int64_t)h * Dv, *a2 = m2 + n * ld + (int64_t)h * Dv;
     float ss = 0.f;
     for (int d = lane; d < Dv; d += 64) { const float o = a1[d] - lambda * a2[d]; ss += o * o; }
     ss = wave_sum_f32(ss);
@@ -68,12 +71,12 @@ __global__ __launch_bounds__(256) void diff_combine_kernel(const float *__restri
     for (int d = lane; d < Dv; d += 64) st_f(out + vec * Dv + d, (a1[d] - lambda * a2[d]) * r);
 }
 
-extern "C" int jl_diff_combine(const float *a, int64_t N, int32_t H, int32_t Dv, float lambda, float eps, float out_scale, void *out,
-                               int dtype, void *stream) {
+extern "C" int jl_diff_combine(const float *a1, const float *a2, int64_t ld, int64_t N, int32_t H, int32_t Dv, float lambda, float eps,
+                               float out_scale, void *out, int dtype, void *stream) {
     if (N <= 0) return JL_OK;
-    if (!a || !out || H <= 0 || Dv <= 0) return jl_fail(JL_E_INVALID, "jl_diff_combine: null pointer or bad sizes");
+    if (!a1 || !a2 || !out || H <= 0 || Dv <= 0 || ld < (int64_t)H * Dv) return jl_fail(JL_E_INVALID, "jl_diff_combine: null pointer or bad sizes");
     const int64_t vecs = N * H;
-    JL_DISPATCH(dtype, diff_combine_kernel<T><<<dim3((unsigned)((vecs + 3) / 4)), 256, 0, (hipStream_t)stream>>>(a, N, H, Dv, lambda, eps, out_scale,
+    JL_DISPATCH(dtype, diff_combine_kernel<T><<<dim3((unsigned)((vecs + 3) / 4)), 256, 0, (hipStream_t)stream>>>(a1, a2, ld, N, H, Dv, lambda, eps, out_scale,
                                                                                                                (T *)out));
     return jl_check_launch("diff_combine_kernel");
 }

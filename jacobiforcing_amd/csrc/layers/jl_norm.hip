@@ -1,22 +1,6 @@
-// jl_norm.hip — error plumbing of libjf_layers.so, embedding gather and the residual-update + RMS-norm launch.
+// jl_norm.hip — embedding gather, the residual-update + RMS-norm launches (norm of the stream, norm of a sublayer's output) and the
+// polynomial activation.
 #include "jl_common.h"
-
-static thread_local char g_err[512] = "";
-
-int jl_fail(int code, const char *fmt, ...) {
-    va_list ap;
-    va_start(ap, fmt);
-    vsnprintf(g_err, sizeof g_err, fmt, ap);
-    va_end(ap);
-    return code;
-}
-int jl_check_launch(const char *what) {
-    hipError_t e = hipGetLastError();
-    if (e != hipSuccess) return jl_fail(JL_E_LAUNCH, "%s: %s", what, hipGetErrorString(e));
-    return JL_OK;
-}
-extern "C" int jl_version(void) { return JL_VERSION; }
-extern "C" const char *jl_last_error(void) { return g_err; }
 
 template <typename T>
 __global__ __launch_bounds__(256) void embed_scale_kernel(const T *__restrict__ embed, const int64_t *__restrict__ ids, int W,

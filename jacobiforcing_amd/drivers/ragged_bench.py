@@ -1,8 +1,9 @@
 #!/usr/bin/env python3
-"""Prefill and decode throughput of a ragged model family (Lokizen) at sizes that resemble a real model's layers, beside the
-package's Qwen2 forward at equal width, depth, head sizes and active feed-forward width — random weights, synthetic tokens.
+"""Prefill and decode throughput of a ragged model family (Lokizen, Vumalix) at sizes that resemble a real model's layers, beside
+the package's closest existing model at equal width, depth, head sizes and active feed-forward width (Lokizen beside Qwen2;
+Vumalix beside Lokizen and Qwen2) — random weights, synthetic tokens.
 
-    python -m jacobiforcing_amd.drivers.ragged_bench [--sizes small,medium] [--kernels]
+    python -m jacobiforcing_amd.drivers.ragged_bench [--design lokizen|vumalix] [--sizes small,medium] [--kernels]
     python bench.py --design lokizen            (the same, as one JSON line)
 
 Per size: prefill = whole prompts in one step (tokens / s), decode = one token for each of ``--decode-batch`` requests at a
@@ -58,11 +59,44 @@ def timed(fn, warmup=2, iters=5):
     return (time.perf_counter() - t0) / iters
 
 
+# Vumalix at the same widths, depths and head counts: latent attention and differential attention alternate; the differential
+# maps have half of Lokizen's head size each, the latent has the rank of a head; the dense feed-forward has the experts' active width
+VSIZES = {
+    "small": dict(width=1024, layers=4, heads=8, kv=2, dim=64, vdim=128, lheads=8, ldim=64, rot=32, lvdim=64, kv_rank=128, q_rank=384,
+                  window=1024, ff=2048, taps=4, vocab=32000),
+    "medium": dict(width=2048, layers=8, heads=16, kv=4, dim=64, vdim=128, lheads=16, ldim=128, rot=64, lvdim=128, kv_rank=512, q_rank=768,
+                   window=2048, ff=4096, taps=4, vocab=32000),
+}
+
+
+def vumalix_config(s):
+    from ..modeling.vumalix import VumalixConfig
+    mlp = {"kind": "dense", "ff": s["ff"]}
+    lat = {"type": "latent_attention", "mlp": mlp,
+           "mixer": {"heads": s["lheads"], "dim": s["ldim"], "rot_dim": s["rot"], "vdim": s["lvdim"], "kv_rank": s["kv_rank"], "q_rank": s["q_rank"],
+                     "scale": (s["ldim"] + s["rot"]) ** -0.5, "mask": {"size": s["window"]}, "rot": {"dims": s["rot"], "base": 1e6}}}
+    att = {"type": "attention", "mlp": mlp, "mixer": {"heads": s["heads"], "kv_heads": s["kv"], "dim": s["dim"], "vdim": s["vdim"], "scale": s["dim"] ** -0.5,
+                                                       "diff": 0.3, "q_temp": {"coef": 0.1, "every": 256}}}
+    return VumalixConfig.from_dict({"architecture": "Vumalix", "vocab": s["vocab"], "width": s["width"], "norm": {"eps": 1e-6}, "canon": {"taps": s["taps"]},
+                                    "layers": [lat if i % 2 == 0 else att for i in range(s["layers"])]})
+
+
 def bench_lokizen(s, prompts, prompt_len, decode_batch, context, dtype=torch.bfloat16):
-    from .. import layer_ops as LO
     from ..modeling.lokizen import random_model
+    model = random_model(lokizen_config(s), "cuda", dtype, max_positions=max(prompt_len, context) + 64)
+    return bench_ragged(model, s["vocab"], prompts, prompt_len, decode_batch, context)
+
+
+def bench_vumalix(s, prompts, prompt_len, decode_batch, context, dtype=torch.bfloat16):
+    from ..modeling.vumalix import random_model
+    model = random_model(vumalix_config(s), "cuda", dtype, max_positions=max(prompt_len, context) + 64)
+    return bench_ragged(model, s["vocab"], prompts, prompt_len, decode_batch, context)
+
+
+def bench_ragged(model, vocab, prompts, prompt_len, decode_batch, context):
+    from .. import layer_ops as LO
     dev = "cuda"
-    model = random_model(lokizen_config(s), dev, dtype, max_positions=max(prompt_len, context) + 64)
+    s = {"vocab": vocab}
     page = 64
     per = -(-(max(prompt_len, context) + 1) // page)
     slots = max(prompts, decode_batch)
@@ -168,7 +202,122 @@ def kernel_table(s, prompts, prompt_len, decode_batch, context, dtype=torch.bflo
     return out
 
 
-def run(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, context=2048, kernels=True):
+def kernel_table_vumalix(s, prompts, prompt_len, decode_batch, context, dtype=torch.bfloat16):
+    """Vumalix's layer kernels alone at the size's shapes, prefill and decode, each beside the like kernel of the closest model
+    (Lokizen's windowed attention, its residual + norm launch, its whole-projection q/k norm; Qwen2's SwiGLU launch)."""
+    from .. import layer_ops as LO
+    from .. import ops
+    dev = "cuda"
+    W, H, G, D, Dv, ff, win, taps = s["width"], s["heads"], s["kv"], s["dim"], s["vdim"], s["ff"], s["window"], s["taps"]
+    LH, LD, rd, LDv, R, Rq = s["lheads"], s["ldim"], s["rot"], s["lvdim"], s["kv_rank"], s["q_rank"]
+    lk = SIZES_BY_WIDTH[W]
+    KH, KG, KD = lk["heads"], lk["kv"], lk["dim"]
+    page, es = 64, 2
+    per = -(-(max(prompt_len, context) + 1) // page)
+    slots = max(prompts, decode_batch)
+    tables = [list(range(b * per, (b + 1) * per)) for b in range(slots)]
+    g = torch.Generator().manual_seed(0)
+    rnd = lambda *sh: torch.randn(*sh, generator=g).to(dev).to(dtype)
+    tokens = slots * per * page
+    kd, vd, lat = rnd(tokens, 2 * G * D), rnd(tokens, G * Dv), rnd(tokens, R + rd)
+    kk, vk = rnd(tokens, KG * KD), rnd(tokens, KG * KD)
+    a = torch.arange(max(prompt_len, context) + 8, dtype=torch.float32, device=dev).view(-1, 1) * torch.rand(rd // 2, device=dev).view(1, -1)
+    cos, sin = a.cos().contiguous(), a.sin().contiguous()
+    tail = torch.zeros((slots, taps - 1, W), device=dev)
+    out = {}
+
+    def row(name, secs, nbytes, flops, peak):
+        bound = max(nbytes / HBM_BPS, flops / peak)
+        out[name] = {"us": round(1e6 * secs, 1), "MB": round(nbytes / 1e6, 2), "GFLOP": round(flops / 1e9, 2), "roofline_fraction": round(bound / secs, 4)}
+
+    for phase, B, T, start in (("prefill", prompts, prompt_len, 0), ("decode", decode_batch, 1, context)):
+        n = B * T
+        batch = LO.RaggedBatch.build([T] * B, [start] * B, list(range(B)), tables[:B], page, dev)
+        causal = B * sum(start + t + 1 for t in range(T))                                       # visible (query, key) pairs per head, no window
+        windowed = B * sum(min(start + t + 1, win) for t in range(T))
+        span_c, span_w = B * (start + T), B * min(start + T, win + T)                              # pool rows a launch has to read once
+        x, y, gw, wn = torch.randn(n, W, device=dev), rnd(n, W), torch.ones(1, device=dev), rnd(W)
+        row(f"{phase}.norm_add", timed(lambda: LO.norm_add(x, y, gw, 1e-6, dtype)), n * W * (4 + 4 + es + es), 4.0 * n * W, VECTOR_FLOPS)
+        row(f"{phase}.lokizen.add_rmsnorm", timed(lambda: LO.add_rmsnorm(x, y, None, wn, 1e-5, dtype)), n * W * (4 + 4 + es + es), 4.0 * n * W, VECTOR_FLOPS)
+        cw = rnd(W, taps)
+        row(f"{phase}.causal_conv", timed(lambda: LO.causal_conv(x, cw, batch, tail)), n * W * (4 + es), 2.0 * taps * n * W, VECTOR_FLOPS)
+        z, coef = rnd(n, ff), torch.tensor([0.5, 0.3, 0.2, 0.1], device=dev)
+        row(f"{phase}.polynorm", timed(lambda: LO.polynorm(z, coef, 1e-6)), 3 * n * ff * es, 12.0 * n * ff, VECTOR_FLOPS)
+        gu = rnd(n, 2 * ff)
+        row(f"{phase}.qwen2.swiglu", timed(lambda: ops.swiglu(gu)), 3 * n * ff * es, 4.0 * n * ff, VECTOR_FLOPS)
+        # differential attention: norm + append, both maps' attention, combination
+        proj = rnd(n, 2 * H * D + 2 * G * D + G * Dv)
+        wq = rnd(D)
+        apart = 2 * H > LO.ATTN_MAX_HEADS_ONE_LAUNCH
+        t_hn = timed(lambda: LO.head_norm_append(proj, (0, 2 * H * D, 2 * H * D + 2 * G * D), H, G, 2, D, Dv, wq, wq, 1e-6, 0.1, 256, batch, kd, vd, apart))
+        row(f"{phase}.head_norm_append", t_hn, 2 * n * (2 * H * D + 2 * G * D + G * Dv) * es, 6.0 * n * (2 * H + 2 * G) * D, VECTOR_FLOPS)
+        pk = rnd(n, KH * KD + 2 * KG * KD)
+        wqk, wkk = rnd(KH * KD), rnd(KG * KD)
+        t_qk = timed(lambda: LO.qk_norm_append(pk, (0, KH * KD, KH * KD + KG * KD), KH, KG, KD, KD, wqk, wkk, 1e-5, kk, vk, batch.kv_slot))
+        row(f"{phase}.lokizen.qk_norm_append", t_qk, 2 * n * (KH * KD + 2 * KG * KD) * es, 6.0 * n * (KH + KG) * KD, VECTOR_FLOPS)
+        q = LO.head_norm_append(proj, (0, 2 * H * D, 2 * H * D + 2 * G * D), H, G, 2, D, Dv, wq, wq, 1e-6, 0.1, 256, batch, kd, vd, apart)
+
+        def diff_attn():
+            if not apart:
+                return LO.attn_window(q, None, kd, vd, batch, 2 * H, 2 * G, D, Dv, D ** -0.5, 0, 0, None, None, None, value_heads=G, float_out=True)
+            return [LO.attn_window(q[mp], None, kd[:, mp * G * D:(mp + 1) * G * D], vd, batch, H, G, D, Dv, D ** -0.5, 0, 0, None, None, None, float_out=True)
+                    for mp in range(2)]
+        row(f"{phase}.attn_differential", timed(diff_attn), span_c * (2 * G * D + G * Dv) * es + n * 2 * H * (D * es + Dv * 4),
+            2.0 * causal * 2 * H * (D + Dv), MATRIX_FLOPS)
+        a12 = torch.randn(n, 2 * H * Dv, device=dev)
+        row(f"{phase}.diff_combine", timed(lambda: LO.diff_combine(a12[:, :H * Dv], a12[:, H * Dv:], H, Dv, 0.4, 1e-6, 0.7, dtype)),
+            n * H * Dv * (8 + es), 6.0 * n * H * Dv, VECTOR_FLOPS)
+        # latent attention: norms + rotation + append, query packing, attention over the latent pool, gate
+        pl = rnd(n, Rq + R + rd + LH * LDv)
+        wlq, wlk = rnd(Rq), rnd(R)
+        t_lp = timed(lambda: LO.latent_prep(pl, 0, Rq, Rq, R, rd, rd, wlq, wlk, 1e-6, batch, cos, sin, lat))
+        row(f"{phase}.latent_prep", t_lp, 2 * n * (Rq + R + rd) * es, 6.0 * n * (Rq + R + rd), VECTOR_FLOPS)
+        qa, ql = rnd(LH, n, R), rnd(n, LH * (LD + rd))
+        row(f"{phase}.latent_q_pack", timed(lambda: LO.latent_q_pack(qa, ql, LH, LD, R, rd, rd, batch, cos, sin)), 2 * n * LH * (R + rd) * es,
+            6.0 * n * LH * rd, VECTOR_FLOPS)
+        qf = LO.latent_q_pack(qa, ql, LH, LD, R, rd, rd, batch, cos, sin)
+        step = LO.ATTN_MAX_VALUE_WIDTH
+
+        def latent_attn():
+            if LO.attn_shared_kv_tile_rows(dtype, LH, R + rd, R, lat.stride(0)):
+                return LO.attn_shared_kv(qf, lat, batch, LH, R + rd, R, 0.1, win)
+            return [LO.attn_window(qf, None, lat, lat[:, c0:min(R, c0 + step)], batch, LH, 1, R + rd, min(R, c0 + step) - c0, 0.1, win, 0, None, None, None)
+                    for c0 in range(0, R, step)]
+        row(f"{phase}.attn_latent", timed(latent_attn), span_w * (R + rd) * es + n * LH * (2 * R + rd) * es, 2.0 * windowed * LH * (2 * R + rd), MATRIX_FLOPS)
+        ov = rnd(LH, n, LDv)
+        row(f"{phase}.heads_gate", timed(lambda: LO.heads_gate(ov, pl[:, Rq + R + rd:])), 3 * n * LH * LDv * es, 6.0 * n * LH * LDv, VECTOR_FLOPS)
+        # the like kernel of the closest model: Lokizen's windowed attention with its bias, head mixing and gate, at its own sizes
+        ql2, gate = rnd(n, KH * KD), rnd(n, KH * KD)
+        rel, talk = torch.randn(max(prompt_len, context) + 8, KH, device=dev), torch.eye(KH, device=dev)
+        t_att = timed(lambda: LO.attn_window(ql2, gate, kk, vk, batch, KH, KG, KD, KD, KD ** -0.5, win, 4, rel, None, talk))
+        row(f"{phase}.lokizen.attn_window", t_att, span_w * 2 * KG * KD * es + 3 * n * KH * KD * es, 4.0 * windowed * KH * KD, MATRIX_FLOPS)
+    return out
+
+
+SIZES_BY_WIDTH = {v["width"]: v for v in SIZES.values()}
+
+
+def run_vumalix(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, context=2048, kernels=True):
+    res = {"bench": "ragged_family", "design": "Vumalix", "closest": "Lokizen", "dtype": "bf16", "data": "synthetic", "prompts": prompts,
+           "prompt_len": prompt_len, "decode_batch": decode_batch, "context": context, "sizes": {}}
+    for name in sizes:
+        s = VSIZES[name]
+        entry = {"shape": s, "vumalix": bench_vumalix(s, prompts, prompt_len, decode_batch, context)}
+        torch.cuda.empty_cache()
+        entry["lokizen"] = bench_lokizen(SIZES[name], prompts, prompt_len, decode_batch, context)
+        torch.cuda.empty_cache()
+        entry["qwen2"] = bench_qwen2(dict(SIZES[name], top=1, ff=s["ff"]), prompts, prompt_len, decode_batch, context)
+        torch.cuda.empty_cache()
+        if kernels:
+            entry["kernels"] = kernel_table_vumalix(s, prompts, prompt_len, decode_batch, context)
+            torch.cuda.empty_cache()
+        res["sizes"][name] = entry
+    return res
+
+
+def run(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, context=2048, kernels=True, design="lokizen"):
+    if design.lower() == "vumalix":
+        return run_vumalix(sizes, prompts, prompt_len, decode_batch, context, kernels)
     res = {"bench": "ragged_family", "design": "Lokizen", "closest": "Qwen2", "dtype": "bf16", "data": "synthetic", "prompts": prompts,
            "prompt_len": prompt_len, "decode_batch": decode_batch, "context": context, "sizes": {}}
     for name in sizes:
@@ -186,6 +335,7 @@ def run(sizes=("small", "medium"), prompts=4, prompt_len=2048, decode_batch=32, 
 
 def main(argv=None):
     ap = argparse.ArgumentParser(description=__doc__.split("\n")[0])
+    ap.add_argument("--design", default="lokizen", choices=("lokizen", "vumalix"))
     ap.add_argument("--sizes", default="small,medium")
     ap.add_argument("--prompts", type=int, default=4)
     ap.add_argument("--prompt-len", type=int, default=2048)
@@ -193,7 +343,7 @@ def main(argv=None):
     ap.add_argument("--context", type=int, default=2048)
     ap.add_argument("--no-kernels", action="store_true")
     a = ap.parse_args(argv)
-    print(json.dumps(run(tuple(a.sizes.split(",")), a.prompts, a.prompt_len, a.decode_batch, a.context, not a.no_kernels)), flush=True)
+    print(json.dumps(run(tuple(a.sizes.split(",")), a.prompts, a.prompt_len, a.decode_batch, a.context, not a.no_kernels, a.design)), flush=True)
 
 
 if __name__ == "__main__":

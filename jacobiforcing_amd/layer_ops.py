@@ -6,6 +6,7 @@ records and tiles the kernels read."""
 from __future__ import annotations
 
 import ctypes as C
+import os
 from dataclasses import dataclass
 from typing import List, Optional, Sequence, Tuple
 
@@ -16,6 +17,7 @@ from . import _native as N
 
 
 ATTN_SPLIT_BELOW_TILES, ATTN_SPLIT_WORKGROUPS = 128, 512     # attention: split a tile's keys while tiles x splits stays below ~2 per CU
+ATTN_MAX_HEADS_ONE_LAUNCH, ATTN_MAX_VALUE_WIDTH = 16, 128   # what the matrix-core attention kernel takes in one workgroup
 RETENTION_CHUNK = 64          # tokens per chunk when a long portion's recurrence is cut into chunks that run side by side
 
 
@@ -230,6 +232,41 @@ def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Te
     return out
 
 
+def attn_shared_kv_tile_rows(dtype: torch.dtype, H: int, D: int, Dv: int, k_ld: int) -> int:
+    """Queries per tile of the shared key/value-head kernel for these sizes; 0 when it does not take them."""
+    if dtype != torch.bfloat16 or os.environ.get("JL_ATTN_NO_SHARED_KV"):                      # A/B switch for measurements
+        return 0
+    return int(N.layers().jl_attn_shared_kv_tile_rows(_code(dtype), H, D, Dv, k_ld))
+
+
+def attn_shared_kv(q: torch.Tensor, pool: torch.Tensor, batch: RaggedBatch, H: int, D: int, Dv: int, scale: float, window: int) -> torch.Tensor:
+    """Attention of H query heads over one key/value head: q [N, H*D]; pool [tokens, >= D] whose rows hold the key (D columns)
+    with the value as its first Dv columns.  Returns [N, H*Dv].  Sizes as ``attn_shared_kv_tile_rows`` accepts them."""
+    _dev(q)
+    n = q.shape[0]
+    _need(q.is_contiguous() and q.shape[1] == H * D and n == batch.N and pool.dtype == q.dtype and pool.dim() == 2 and pool.stride(1) == 1 and
+          pool.shape[1] >= D and Dv <= D, "attn_shared_kv: q [N, H*D] of the batch, pool rows of at least D columns")
+    _need(pool.shape[0] % batch.page_size == 0 and batch.max_page < pool.shape[0] // batch.page_size, "attn_shared_kv: a page lies outside the pool")
+    tq = attn_shared_kv_tile_rows(q.dtype, H, D, Dv, pool.stride(0))
+    _need(tq > 0, f"attn_shared_kv: heads={H} dim={D} vdim={Dv} are not sizes of this kernel")
+    tiles = batch.tiles(tq)
+    out = torch.empty((n, H * Dv), dtype=q.dtype, device=q.device)
+    # few tiles with many keys (decoding): share each tile's keys out over workgroups until the chip is full
+    groups = tiles.shape[0] * -(-H // 32)
+    splits, scratch = 1, None
+    if groups < ATTN_SPLIT_BELOW_TILES:
+        reach = batch.max_pos if window <= 0 else min(batch.max_pos, int(window) + tq)
+        splits = max(1, min(-(-reach // 64), ATTN_SPLIT_WORKGROUPS // groups, 64))
+        if splits > 1:
+            scratch = torch.empty((int(N.layers().jl_attn_shared_kv_scratch_floats(tiles.shape[0], H, Dv, splits)),), dtype=torch.float32, device=q.device)
+    a = N.AttnArgs(q=q.data_ptr(), k_cache=pool.data_ptr(), v_cache=pool.data_ptr(), out=out.data_ptr(), block_tables=batch.tables.data_ptr(),
+                   tiles=tiles.data_ptr(), bt_stride=batch.tables.shape[1], n_tiles=tiles.shape[0], page_size=batch.page_size, H=H, G=1, D=D, Dv=Dv,
+                   window=int(window), TQ=tq, dtype=_code(q.dtype), scale=float(scale), n_rows=n, k_ld=pool.stride(0), Gv=1, splits=splits,
+                   scratch=scratch.data_ptr() if scratch is not None else None)
+    N.check_layers(N.layers().jl_attn_shared_kv(C.byref(a), _stream(q.device)), "jl_attn_shared_kv")
+    return out
+
+
 def retention(proj: torch.Tensor, cols: Tuple[int, int, int, int], batch: RaggedBatch, H: int, D: int, Dv: int, rot_dims: int,
               cos: Optional[torch.Tensor], sin: Optional[torch.Tensor], decay: torch.Tensor, eps: float, state: torch.Tensor) -> torch.Tensor:
     """proj [N, ld] with q, k, v, gate at ``cols``; state [slots, H, D, Dv] float (updated in place).  Returns [N, H*Dv]."""
@@ -337,15 +374,17 @@ def causal_conv(x: torch.Tensor, w: torch.Tensor, batch: RaggedBatch, tail: Opti
     L, st = N.layers(), _stream(x.device)
     N.check_layers(L.jl_causal_conv(_ptr(x), _ptr(w), _code(w.dtype), _ptr(batch.row_req), _ptr(batch.seq), _ptr(tail), n, W, taps, _ptr(out), st),
                    "jl_causal_conv")
-    if taps > 1:
+    if taps > 1 and max(batch.counts) > 1:                  # single rows (decoding) have moved their tails in the launch above
         N.check_layers(L.jl_causal_conv_carry(_ptr(x), _ptr(batch.seq), batch.B, _ptr(tail), W, taps, st), "jl_causal_conv_carry")
     return out
 
 
 def head_norm_append(proj: torch.Tensor, cols: Tuple[int, int, int], H: int, G: int, M: int, D: int, Dv: int, wq: torch.Tensor, wk: torch.Tensor,
-                     eps: float, t_coef: float, t_every: int, batch: RaggedBatch, k_cache: torch.Tensor, v_cache: torch.Tensor) -> torch.Tensor:
+                     eps: float, t_coef: float, t_every: int, batch: RaggedBatch, k_cache: torch.Tensor, v_cache: torch.Tensor,
+                     maps_apart: bool = False) -> torch.Tensor:
     """Per-head (and per score map) RMS norm of q and k over D, query temperature by position, keys / values appended to the
-    pools.  Returns q [N, M*H*D] map-major; the key pool rows are [M, G, D] map-major."""
+    pools.  Returns q [N, M*H*D] map-major ([M, N, H*D] with ``maps_apart``: a contiguous query matrix per map); the key pool rows
+    are [M, G, D] map-major."""
     _dev(proj)
     n, ld = proj.shape
     dt = proj.dtype
@@ -353,21 +392,23 @@ def head_norm_append(proj: torch.Tensor, cols: Tuple[int, int, int], H: int, G: 
     _need(wq.numel() == D and wk.numel() == D and wq.dtype == dt and wk.dtype == dt, "head_norm_append: norm weights over one head")
     _need(k_cache.dtype == dt and v_cache.dtype == dt and k_cache.is_contiguous() and v_cache.is_contiguous() and
           k_cache.shape[-1] == M * G * D and v_cache.shape[-1] == G * Dv and k_cache.shape[0] == v_cache.shape[0], "head_norm_append: pools [tokens, M*G*D] / [tokens, G*Dv]")
-    q = torch.empty((n, M * H * D), dtype=dt, device=proj.device)
+    q = torch.empty((M, n, H * D) if maps_apart else (n, M * H * D), dtype=dt, device=proj.device)
     N.check_layers(N.layers().jl_head_norm_append(_ptr(proj), _code(dt), n, ld, cols[0], cols[1], cols[2], H, G, M, D, Dv, _ptr(wq), _ptr(wk), float(eps),
-                                                 float(t_coef), int(t_every), _ptr(batch.pos), _ptr(q), _ptr(k_cache), _ptr(v_cache),
+                                                 float(t_coef), int(t_every), _ptr(batch.pos), _ptr(q), int(maps_apart), _ptr(k_cache), _ptr(v_cache),
                                                  _ptr(batch.kv_slot), _stream(proj.device)), "jl_head_norm_append")
     return q
 
 
-def diff_combine(a: torch.Tensor, H: int, Dv: int, lam: float, eps: float, out_scale: float, out_dtype: torch.dtype) -> torch.Tensor:
-    """a float [N, 2*H*Dv] (two score maps' outputs, map-major) -> rms_norm_per_head(a[0] - lam * a[1]) * out_scale, [N, H*Dv]."""
-    _dev(a)
-    n = a.shape[0]
-    _need(a.dtype == torch.float32 and a.is_contiguous() and a.shape[1] == 2 * H * Dv, "diff_combine: a float [N, 2*H*Dv]")
-    out = torch.empty((n, H * Dv), dtype=out_dtype, device=a.device)
-    N.check_layers(N.layers().jl_diff_combine(_ptr(a), n, H, Dv, float(lam), float(eps), float(out_scale), _ptr(out), _code(out_dtype),
-                                             _stream(a.device)), "jl_diff_combine")
+def diff_combine(a1: torch.Tensor, a2: torch.Tensor, H: int, Dv: int, lam: float, eps: float, out_scale: float, out_dtype: torch.dtype) -> torch.Tensor:
+    """a1, a2 float [N, H*Dv] (two score maps' outputs; views with a common row stride) -> rms_norm_per_head(a1 - lam * a2) *
+    out_scale, [N, H*Dv]."""
+    _dev(a1)
+    n = a1.shape[0]
+    _need(a1.dtype == torch.float32 and a2.dtype == torch.float32 and tuple(a1.shape) == (n, H * Dv) and a2.shape == a1.shape and
+          a1.stride(1) == 1 and a2.stride(1) == 1 and a1.stride(0) == a2.stride(0), "diff_combine: two float [N, H*Dv] with one row stride")
+    out = torch.empty((n, H * Dv), dtype=out_dtype, device=a1.device)
+    N.check_layers(N.layers().jl_diff_combine(_ptr(a1), _ptr(a2), a1.stride(0), n, H, Dv, float(lam), float(eps), float(out_scale), _ptr(out),
+                                             _code(out_dtype), _stream(a1.device)), "jl_diff_combine")
     return out
 
 

@@ -224,12 +224,17 @@ class VumalixModel:
         H, G, D, Dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
         qt = m.get("q_temp") or {}
         proj = F.linear(h, w["w_in"])
+        apart = 2 * H > LO.ATTN_MAX_HEADS_ONE_LAUNCH
         q = LO.head_norm_append(proj, w["cols"], H, G, 2, D, Dv, w["q_norm"], w["k_norm"], eps, float(qt.get("coef", 0.0)), int(qt.get("every", 1)),
-                                batch, cache.k[li], cache.v[li])
-        # one launch for both maps: 2H query heads over 2G key heads and G value heads, plain causal, float outputs
-        a = LO.attn_window(q, None, cache.k[li], cache.v[li], batch, 2 * H, 2 * G, D, Dv, float(m["scale"]), 0, 0, None, None, None,
-                           value_heads=G, float_out=True)
-        return LO.diff_combine(a, H, Dv, w["lam"], eps, 1.0 - float(m["diff"]), self.dtype)
+                                batch, cache.k[li], cache.v[li], maps_apart=apart)
+        kp, vp, scale = cache.k[li], cache.v[li], float(m["scale"])
+        if not apart:   # one launch for both maps: 2H query heads over 2G key heads and G value heads, plain causal, float outputs
+            a = LO.attn_window(q, None, kp, vp, batch, 2 * H, 2 * G, D, Dv, scale, 0, 0, None, None, None, value_heads=G, float_out=True)
+            a1, a2 = a[:, :H * Dv], a[:, H * Dv:]
+        else:           # more heads than one workgroup takes: a launch per map over its own columns of the key rows
+            a1, a2 = (LO.attn_window(q[mp], None, kp[:, mp * G * D:(mp + 1) * G * D], vp, batch, H, G, D, Dv, scale, 0, 0, None, None, None,
+                                     float_out=True) for mp in range(2))
+        return LO.diff_combine(a1, a2, H, Dv, w["lam"], eps, 1.0 - float(m["diff"]), self.dtype)
 
     def _latent_attention(self, li: int, h: torch.Tensor, batch: LO.RaggedBatch, cache: PagedStateCache) -> torch.Tensor:
         m, w, eps = self.cfg.layers[li]["mixer"], self.w.layers[li], self.cfg.norm_eps
@@ -244,9 +249,21 @@ class VumalixModel:
         q = F.linear(cq, w["w_uq"])
         qa = torch.bmm(q.view(n, H, D + rd)[:, :, :D].transpose(0, 1), w["w_uk"])                    # [H, N, R]: query . (W_uk c) = (W_uk^T query) . c
         qf = LO.latent_q_pack(qa, q, H, D, R, rd, dims, batch, cos, sin)
-        o = LO.attn_window(qf, None, pool, pool[:, :R], batch, H, 1, R + rd, R, float(m["scale"]), int((m.get("mask") or {}).get("size", 0)), 0,
-                           None, None, None)
-        ov = torch.bmm(o.view(n, H, R).transpose(0, 1), w["w_uv"])                                   # [H, N, Dv]
+        window, scale = int((m.get("mask") or {}).get("size", 0)), float(m["scale"])
+        step = LO.ATTN_MAX_VALUE_WIDTH
+        if LO.attn_shared_kv_tile_rows(self.dtype, H, R + rd, R, pool.stride(0)):                   # bfloat16, latents of 128 .. 512: one sweep
+            o = LO.attn_shared_kv(qf, pool, batch, H, R + rd, R, scale, window)
+            ov = torch.bmm(o.view(n, H, R).transpose(0, 1), w["w_uv"])
+        elif R <= step or self.dtype != torch.bfloat16:
+            o = LO.attn_window(qf, None, pool, pool[:, :R], batch, H, 1, R + rd, R, scale, window, 0, None, None, None)
+            ov = torch.bmm(o.view(n, H, R).transpose(0, 1), w["w_uv"])                               # [H, N, Dv]
+        else:           # a latent wider than the matrix-core kernel's value tile: a launch per column range of the latent
+            ov = None
+            for c0 in range(0, R, step):
+                c1 = min(R, c0 + step)
+                o = LO.attn_window(qf, None, pool, pool[:, c0:c1], batch, H, 1, R + rd, c1 - c0, scale, window, 0, None, None, None)
+                o = o.view(n, H, c1 - c0).transpose(0, 1)
+                ov = torch.bmm(o, w["w_uv"][:, c0:c1]) if ov is None else torch.baddbmm(ov, o, w["w_uv"][:, c0:c1])
         return LO.heads_gate(ov, proj[:, w["cols"][2]:w["cols"][2] + H * Dv])
 
     # ---- one step ----------------------------------------------------------------------------------------------------------------

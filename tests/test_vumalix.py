@@ -370,8 +370,11 @@ def test_bfloat16_differential_attention_alone(H, G, D, Dv):
 
 @gpu
 @pytest.mark.parametrize("H,D,rd,Dv,R,size", [(6, 64, 32, 48, 96, 50), (4, 32, 16, 48, 64, 20), (16, 16, 8, 16, 32, 33), (2, 24, 8, 20, 200, 40),
-                                               (20, 16, 16, 16, 48, 17)])
+                                               (20, 16, 16, 16, 48, 17), (6, 48, 16, 40, 128, 50), (16, 32, 32, 32, 256, 33), (40, 16, 8, 16, 128, 20),
+                                               (3, 24, 8, 20, 384, 70), (1, 16, 64, 24, 512, 1000), (5, 16, 8, 16, 128, 1)])
 def test_bfloat16_latent_attention_alone(H, D, rd, Dv, R, size):
+    """Latents of 128, 256, 384 and 512 take the one-sweep kernel for a shared key/value head (1, 3, 5, 6, 16 and 40 heads: part of
+    a row tile, a whole one, two of them); the others the general kernels, 200 in two column ranges."""
     import torch.nn.functional as F
     cfg = make_cfg([dict(latent(heads=H, dim=D, rot_dim=rd, vdim=Dv, kv_rank=R, q_rank=40, size=size, scale=(D + rd) ** -0.5), mlp=None)], width=64)
     rig = Rig(cfg, seed=H, dtype=torch.bfloat16, page=16)
@@ -424,17 +427,17 @@ def test_freed_pages_and_slots_are_used_again(dtype, tol):
         assert len(rig.free_pages) == 12 and len(used) >= 8
 
 
-def peaked_latent_model(size):
+def peaked_latent_model(size, R=24):
     """One latent-attention layer, no feed-forward, a sharp softmax, a convolution and a rotary part too weak to matter.  Returns
     (cfg, tensors, hot query token, hot key token, scores): the pair of tokens whose unrotated score is the largest."""
-    cfg = make_cfg([dict(latent(heads=2, dim=16, rot_dim=8, vdim=16, kv_rank=24, q_rank=24, size=size, scale=3.0), mlp=None)], width=32, vocab=40)
+    cfg = make_cfg([dict(latent(heads=2, dim=16, rot_dim=8, vdim=16, kv_rank=R, q_rank=24, size=size, scale=3.0), mlp=None)], width=32, vocab=40)
     t = tensors_for(cfg, 23)
     t["l0.canon1"] = t["l0.canon1"] * 0.02
-    t["l0.mix.dkv"][24:] *= 0.05
+    t["l0.mix.dkv"][R:] *= 0.05
     eps = cfg["norm"]["eps"]
     h = t["embed"].double()
     q = ((O.unit_rms(h @ t["l0.mix.dq"].double().T, eps) * t["l0.mix.dq.norm"].double()) @ t["l0.mix.uq"].double().T).view(40, 2, 24)[:, 0, :16]
-    lat = O.unit_rms((h @ t["l0.mix.dkv"].double().T)[:, :24], eps) * t["l0.mix.dkv.norm"].double()
+    lat = O.unit_rms((h @ t["l0.mix.dkv"].double().T)[:, :R], eps) * t["l0.mix.dkv.norm"].double()
     s = q @ (lat @ t["l0.mix.uk"].double().T)[:, :16].T
     qi, kj = divmod(int(s.argmax()), 40)
     return cfg, t, qi, kj, s
@@ -442,10 +445,10 @@ def peaked_latent_model(size):
 
 @gpu
 @pytest.mark.parametrize("decode", [False, True])
-@pytest.mark.parametrize("dtype,tol", [(torch.float32, F32_TOL), (torch.bfloat16, BF16_TOL)])
-def test_a_key_just_inside_and_just_outside_the_window(decode, dtype, tol):
+@pytest.mark.parametrize("dtype,tol,R", [(torch.float32, F32_TOL, 24), (torch.bfloat16, BF16_TOL, 24), (torch.bfloat16, BF16_TOL, 128)])
+def test_a_key_just_inside_and_just_outside_the_window(decode, dtype, tol, R):
     size = 21
-    cfg, t, qi, kj, s = peaked_latent_model(size)
+    cfg, t, qi, kj, s = peaked_latent_model(size, R)
     dull = [x for x in np.argsort(s[qi].numpy())[:12].tolist() if x != kj]                         # keys the hot query ignores
     T = 70
     cases = {"window_in": T - 1 - (size - 1), "window_out": T - 1 - size, "page_border_in": 56, "first": 0, "near": T - 2}
