@@ -74,15 +74,17 @@ JL_API int jl_attn_window(const jl_attn_args *a, void *stream);
  * they do not fit */
 JL_API int jl_attn_tile_rows(int dtype, int32_t H, int32_t G, int32_t D, int32_t Dv, int64_t k_ld, int64_t v_ld);
 
-/* The same attention for ONE key/value head shared by all H query heads whose values are the first Dv columns of the key rows (the
- * pool of latent attention), on the matrix cores in one sweep: bfloat16, G = 1, D % 8 == 0 up to 640, Dv in {128, 256, 384, 512} <= D,
- * k_ld % 4 == 0; no bias, head mixing or gate.  Of jl_attn_args it reads q, k_cache, k_ld, out, block_tables, bt_stride, tiles, n_tiles,
- * page_size, H, G, D, Dv, window, scale, dtype and TQ, which must be what jl_attn_shared_kv_tile_rows returns (0: sizes not taken). */
-JL_API int jl_attn_shared_kv(const jl_attn_args *a, void *stream);
-JL_API int jl_attn_shared_kv_tile_rows(int dtype, int32_t H, int32_t D, int32_t Dv, int64_t k_ld);
-/* splits in 2 .. 64: the keys of every tile are shared out over that many workgroups and joined by a second launch; `scratch` then
- * holds this many floats */
-JL_API int64_t jl_attn_shared_kv_scratch_floats(int32_t n_tiles, int32_t H, int32_t Dv, int32_t splits);
+/* The same attention without bias, head mixing and gate, in ONE sweep over the keys on the matrix cores, for heads in groups that
+ * share a key head (H / G query heads per key head c, value head c % Gv): bfloat16, D % 8 == 0 up to 640, Dv % 32 == 0 up to 512,
+ * row strides % 4 == 0.  v_cache == k_cache (with G = 1, Dv <= D): the values are the first Dv columns of the key rows — the pool
+ * of latent attention — and are not loaded a second time.  Of jl_attn_args it reads q, k_cache, v_cache, k_ld, v_ld, out, out_dtype,
+ * block_tables, bt_stride, tiles, n_tiles, page_size, H, G, Gv, D, Dv, window, scale, dtype, splits, scratch and TQ, which must be
+ * what jl_attn_sweep_tile_rows returns (0: sizes not taken).  splits in 2 .. 64: the keys of every tile are shared out over that
+ * many workgroups and joined by a second launch; `scratch` then holds jl_attn_sweep_scratch_floats floats. */
+JL_API int jl_attn_sweep(const jl_attn_args *a, void *stream);
+JL_API int jl_attn_sweep_tile_rows(int dtype, int32_t H, int32_t G, int32_t Gv, int32_t D, int32_t Dv, int64_t k_ld, int64_t v_ld,
+                                   int32_t v_in_k);
+JL_API int64_t jl_attn_sweep_scratch_floats(int32_t n_tiles, int32_t H, int32_t G, int32_t Dv, int32_t splits);
 
 /* Sublayer-output norm + residual update: x[n] += y[n] / sqrt(mean(y[n]^2) + eps) * g[0] (x float in place, y of y_dtype, g one
  * float); when `out` is given, out[n] = x[n] in `out_dtype` (what the next sublayer's product reads). */

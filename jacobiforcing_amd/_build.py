@@ -20,7 +20,7 @@ HIP_FLAGS = ["--offload-arch=gfx950", "-O3", "-std=c++17", "-fPIC", "-fvisibilit
 # The layer kernels come in two libraries, so that a model compiles (at the first call of a fresh checkout) only what it launches:
 # "layers" = norms, convolution, attention and its input / output stages; "layers_seq" = the recurrent mixer and the routed experts.
 LAYER_GROUPS = {
-    "layers": ["jl_error", "jl_norm", "jl_conv", "jl_headnorm", "jl_latent", "jl_attn_shared", "jl_attn"],
+    "layers": ["jl_error", "jl_norm", "jl_conv", "jl_headnorm", "jl_latent", "jl_attn_sweep", "jl_attn"],
     "layers_seq": ["jl_error", "jl_retention", "jl_moe"],
 }
 LAYERS_HEADERS = [CSRC / "layers" / "jl_common.h", ROOT / "include" / "jf_layers.h"]

@@ -1,16 +1,18 @@
-// jl_attn_shared.hip — attention over ONE key/value head shared by all query heads, whose values are the first Dv columns of the key
-// rows (the pool of latent attention: [latent | rotary key]), on the matrix cores (bfloat16).  Sliding window or plain causal, one
-// sweep with a running maximum and sum.
+// jl_attn_sweep.hip — attention in ONE sweep over the keys (running maximum and sum) on the matrix cores (bfloat16), for heads that
+// come in groups sharing a key head: grouped-query attention, several score maps over the same values, and the single key/value
+// head of latent attention whose values are the first Dv columns of the key rows ([latent | rotary key]).  Sliding window or plain
+// causal; no bias, head mixing or gate (those are jl_attn.hip's).
 //
-// A workgroup of four wavefronts owns up to 32 rows = (query, head) pairs of one request — HF = min(H, 32) heads of 32 / HF
-// consecutive queries — and walks the visible keys 32 at a time through LDS.  Per key tile:
+// A workgroup of four wavefronts owns up to 32 rows = (query, head) pairs of one request and one group — HF = min(heads per group,
+// 32) heads of 32 / HF consecutive queries — so a key tile (32 keys through LDS) serves every head of the group at once.  Per tile:
 //   1. the four wavefronts each form the 32 x 32 scores over a quarter of the key width (v_mfma_f32_32x32x8_bf16; the query
 //      fragments stay in registers for the whole launch) and leave their partial sums in LDS;
 //   2. 8 threads per row add the partial sums, mask, update the row's maximum and sum, and write exp(s - max) as bfloat16 and the
 //      rescale factor of the row;
-//   3. every wavefront multiplies the weights with ITS quarter of the value columns (the same LDS rows the keys were read from).
+//   3. every wavefront multiplies the weights with ITS 32-column tiles of the values (tile wave, wave + 4, ..), which sit in LDS
+//      beside the keys — or ARE the keys' first columns.
 // Few tiles with many keys (decoding): the key tiles of a row tile are shared out over blockIdx.z; every share leaves its
-// unnormalised outputs with its maximum and sum in a scratch, and attn_shared_join_kernel combines them.
+// unnormalised outputs with its maximum and sum in a scratch, and attn_sweep_join_kernel combines them.
 // Accumulator r of lane l of a 32 x 32 MFMA is row 8 * (r / 4) + 4 * (l / 32) + r % 4, column l % 32; lane l supplies row (A) or
 // column (B) l % 32 with depths 4 * (l / 32) .. + 3.
 #include "jl_common.h"
@@ -26,19 +28,23 @@ __device__ __forceinline__ short as_bf16(float v) {
     return (short)(u >> 16);
 }
 
-static size_t as_lds_bytes(int D) { return (size_t)AS_T * (D + 4) * 2 + (size_t)AS_WAVES * AS_T * 33 * 4 + (size_t)AS_T * AS_PROW * 2 + 2 * AS_T * 4; }
+static size_t as_lds_bytes(int D, int Dv, bool v_in_k) {
+    return (size_t)AS_T * (D + 4) * 2 + (v_in_k ? 0 : (size_t)AS_T * (Dv + 4) * 2) + (size_t)AS_WAVES * AS_T * 33 * 4 + (size_t)AS_T * AS_PROW * 2 + 2 * AS_T * 4;
+}
 
-template <int NT>                                                                       // value columns per wavefront = 32 * NT, Dv = 128 * NT
-__global__ __launch_bounds__(AS_THREADS) void attn_shared_kv_kernel(jl_attn_args a, int HF, int TQ) {
+template <int NT>                                                                       // value tiles (32 columns) per wavefront: Dv <= 128 * NT
+__global__ __launch_bounds__(AS_THREADS) void attn_sweep_kernel(jl_attn_args a, int HF, int TQ, int HB, int v_in_k) {
     extern __shared__ __attribute__((aligned(16))) char smem[];
-    const int H = a.H, D = a.D, Dv = a.Dv, KROW = D + 4;
+    const int H = a.H, D = a.D, Dv = a.Dv, KROW = D + 4, VROW = v_in_k ? KROW : Dv + 4, per_group = H / a.G;
     const int tid = threadIdx.x, wave = tid >> 6, lane = tid & 63, l32 = lane & 31, hi = lane >> 5;
     const int *tile = a.tiles + 4 * (int64_t)blockIdx.x;
     const int b = tile[0], i0 = tile[1], cnt = tile[2], row0 = tile[3];
     if (b < 0 || cnt <= 0) return;
-    const int h0 = blockIdx.y * HF;
+    const int c = blockIdx.y / HB;                                  // the group = key head; its query heads are c * per_group ..
+    const int h0 = c * per_group + (blockIdx.y - c * HB) * HF, h_end = (c + 1) * per_group;
     bf16_t *Ks = (bf16_t *)smem;                                    // [32][D + 4]
-    float *Sp = (float *)(Ks + AS_T * KROW);                        // [4][32][33] partial scores
+    bf16_t *Vs = v_in_k ? Ks : Ks + AS_T * KROW;                    // [32][Dv + 4], or the keys' own rows
+    float *Sp = (float *)(Vs + (v_in_k ? AS_T * KROW : AS_T * VROW));   // [4][32][33] partial scores
     bf16_t *Pb = (bf16_t *)(Sp + AS_WAVES * AS_T * 33);             // [32][36] weights
     float *alphaS = (float *)(Pb + AS_T * AS_PROW);                 // [32] rescale factor of the tile
     float *lS = alphaS + AS_T;                                      // [32] final sums
@@ -47,14 +53,15 @@ __global__ __launch_bounds__(AS_THREADS) void attn_shared_kv_kernel(jl_attn_args
     const int lo = i0 - window + 1 > 0 ? i0 - window + 1 : 0;
     const int n_keys = i_max + 1 - lo;
     const int *bt = a.block_tables + (int64_t)b * a.bt_stride;
-    const bf16_t *kc = (const bf16_t *)a.k_cache;
+    const bf16_t *kc = (const bf16_t *)a.k_cache + (int64_t)c * D;
+    const bf16_t *vc = (const bf16_t *)a.v_cache + (int64_t)(c % a.Gv) * Dv;
     const int page_shift = (a.page_size & (a.page_size - 1)) == 0 ? __builtin_ctz(a.page_size) : -1;
 
     // this lane's query fragments: row l32 = (query l32 / HF, head h0 + l32 % HF), key-width steps wave, wave + 4, ..
     as_bf16x4 qf[AS_QSTEPS];
     {
         const int ii = l32 / HF, hh = h0 + l32 % HF;
-        const bool ok = l32 < TQ * HF && ii < cnt && hh < H;
+        const bool ok = l32 < TQ * HF && ii < cnt && hh < h_end;
         const bf16_t *qp = (const bf16_t *)a.q + ((int64_t)(row0 + ii) * H + hh) * D + 4 * hi;
 #pragma unroll
         for (int x = 0; x < AS_QSTEPS; ++x) {
@@ -66,7 +73,7 @@ __global__ __launch_bounds__(AS_THREADS) void attn_shared_kv_kernel(jl_attn_args
     // the row this thread helps to reduce: row tid / 8, keys 4 * (tid % 8) .. + 3
     const int rr = tid >> 3, rc = (tid & 7) * 4;
     const int r_i = i0 + rr / HF;
-    const bool r_ok = rr < TQ * HF && rr / HF < cnt && h0 + rr % HF < H;
+    const bool r_ok = rr < TQ * HF && rr / HF < cnt && h0 + rr % HF < h_end;
     float m_run = -INFINITY, l_run = 0.f;
 
     as_f32x16 acc[NT];
@@ -77,6 +84,8 @@ __global__ __launch_bounds__(AS_THREADS) void attn_shared_kv_kernel(jl_attn_args
 
     const int units = D / 4;                                        // 8-byte units per key row
     const int jj0 = tid / units, u0r = tid - jj0 * units, dj = AS_THREADS / units, dr = AS_THREADS - dj * units;
+    const int vunits = Dv / 4;
+    const int vj0 = tid / vunits, v0r = tid - vj0 * vunits, vdj = AS_THREADS / vunits, vdr = AS_THREADS - vdj * vunits;
 
     const int S = a.splits > 1 ? a.splits : 1, split = blockIdx.z;
     const int per = ((n_keys + AS_T - 1) / AS_T + S - 1) / S;       // key tiles per share
@@ -97,6 +106,21 @@ __global__ __launch_bounds__(AS_THREADS) void attn_shared_kv_kernel(jl_attn_args
                 *(uint2 *)(Ks + jj * KROW + 4 * r) = v;
                 jj += dj; r += dr;
                 if (r >= units) { r -= units; ++jj; }
+            }
+        }
+        if (!v_in_k) {
+            int jj = vj0, r = v0r;
+            for (int e = tid; e < AS_T * vunits; e += AS_THREADS) {
+                uint2 v = make_uint2(0, 0);
+                if (jj < nk) {
+                    const int j = lo + u0 + jj;
+                    const int pg = page_shift >= 0 ? j >> page_shift : j / a.page_size;
+                    const int64_t tok = (int64_t)bt[pg] * a.page_size + (j - pg * a.page_size);
+                    v = *(const uint2 *)(vc + tok * a.v_ld + 4 * r);
+                }
+                *(uint2 *)(Vs + jj * VROW + 4 * r) = v;
+                jj += vdj; r += vdr;
+                if (r >= vunits) { r -= vunits; ++jj; }
             }
         }
         __syncthreads();
@@ -164,8 +188,10 @@ __global__ __launch_bounds__(AS_THREADS) void attn_shared_kv_kernel(jl_attn_args
                 const as_bf16x4 wa = *(const as_bf16x4 *)(Pb + l32 * AS_PROW + j0);
 #pragma unroll
                 for (int t = 0; t < NT; ++t) {
-                    const bf16_t *vp = Ks + j0 * KROW + wave * (32 * NT) + 32 * t + l32;
-                    const as_bf16x4 vb = {(short)vp[0], (short)vp[KROW], (short)vp[2 * KROW], (short)vp[3 * KROW]};
+                    const int col = 32 * (AS_WAVES * t + wave);
+                    if (col >= Dv) continue;
+                    const bf16_t *vp = Vs + j0 * VROW + col + l32;
+                    const as_bf16x4 vb = {(short)vp[0], (short)vp[VROW], (short)vp[2 * VROW], (short)vp[3 * VROW]};
                     acc[t] = __builtin_amdgcn_mfma_f32_32x32x8bf16_1k(wa, vb, acc[t], 0, 0, 0);
                 }
             }
@@ -178,7 +204,8 @@ __global__ __launch_bounds__(AS_THREADS) void attn_shared_kv_kernel(jl_attn_args
         for (int r = 0; r < 16; ++r) {
             const int row = 8 * (r >> 2) + 4 * hi + (r & 3);
 #pragma unroll
-            for (int t = 0; t < NT; ++t) part[row * (Dv + 2) + wave * (32 * NT) + 32 * t + l32] = acc[t][r];
+            for (int t = 0; t < NT; ++t)
+                if (32 * (AS_WAVES * t + wave) < Dv) part[row * (Dv + 2) + 32 * (AS_WAVES * t + wave) + l32] = acc[t][r];
         }
         return;
     }
@@ -189,20 +216,26 @@ __global__ __launch_bounds__(AS_THREADS) void attn_shared_kv_kernel(jl_attn_args
     for (int r = 0; r < 16; ++r) {
         const int row = 8 * (r >> 2) + 4 * hi + (r & 3);
         const int ii = row / HF, hh = h0 + row % HF;
-        if (row >= TQ * HF || ii >= cnt || hh >= H) continue;
+        if (row >= TQ * HF || ii >= cnt || hh >= h_end) continue;
         const float inv = lS[row];
 #pragma unroll
-        for (int t = 0; t < NT; ++t)
-            st_f(out + ((int64_t)(row0 + ii) * H + hh) * Dv + wave * (32 * NT) + 32 * t + l32, acc[t][r] * inv);
+        for (int t = 0; t < NT; ++t) {
+            const int col = 32 * (AS_WAVES * t + wave) + l32;
+            if (col - l32 >= Dv) continue;
+            const int64_t o = ((int64_t)(row0 + ii) * H + hh) * Dv + col;
+            if (a.out_dtype == JL_OUT_F32) ((float *)a.out)[o] = acc[t][r] * inv;
+            else st_f(out + o, acc[t][r] * inv);
+        }
     }
 }
 
 // out[row] = sum_s part_s[row] * exp(m_s - M) / sum_s l_s * exp(m_s - M), in share order
-__global__ __launch_bounds__(256) void attn_shared_join_kernel(jl_attn_args a, int HF, int TQ) {
+__global__ __launch_bounds__(256) void attn_sweep_join_kernel(jl_attn_args a, int HF, int TQ, int HB) {
     __shared__ float wS[AS_T * 64];                                 // [32][S] weight of every share of a row
     const int H = a.H, Dv = a.Dv, S = a.splits, tid = threadIdx.x;
     const int *tile = a.tiles + 4 * (int64_t)blockIdx.x;
-    const int cnt = tile[2], row0 = tile[3], h0 = blockIdx.y * HF;
+    const int cnt = tile[2], row0 = tile[3], per_group = H / a.G, c = blockIdx.y / HB;
+    const int h0 = c * per_group + (blockIdx.y - c * HB) * HF, h_end = (c + 1) * per_group;
     if (tile[0] < 0 || cnt <= 0) return;
     const int64_t share = (int64_t)gridDim.x * gridDim.y * AS_T * (Dv + 2);
     const float *base = a.scratch + ((int64_t)blockIdx.x * gridDim.y + blockIdx.y) * AS_T * (int64_t)(Dv + 2);
@@ -222,59 +255,70 @@ __global__ __launch_bounds__(256) void attn_shared_join_kernel(jl_attn_args a, i
     bf16_t *out = (bf16_t *)a.out;
     for (int e = tid; e < AS_T * Dv; e += 256) {
         const int row = e / Dv, col = e - row * Dv, ii = row / HF, hh = h0 + row % HF;
-        if (row >= TQ * HF || ii >= cnt || hh >= H) continue;
+        if (row >= TQ * HF || ii >= cnt || hh >= h_end) continue;
         float v = 0.f;
         for (int sp = 0; sp < S; ++sp) v += wS[row * 64 + sp] * base[sp * share + row * (Dv + 2) + col];
-        st_f(out + ((int64_t)(row0 + ii) * H + hh) * Dv + col, v);
+        const int64_t o = ((int64_t)(row0 + ii) * H + hh) * Dv + col;
+        if (a.out_dtype == JL_OUT_F32) ((float *)a.out)[o] = v;
+        else st_f(out + o, v);
     }
 }
 
-extern "C" int64_t jl_attn_shared_kv_scratch_floats(int32_t n_tiles, int32_t H, int32_t Dv, int32_t splits) {
-    const int hf = H < AS_T ? H : AS_T;
-    return splits > 1 ? (int64_t)splits * n_tiles * ((H + hf - 1) / hf) * AS_T * (Dv + 2) : 0;
+static int as_heads_per_tile(int H, int G) { const int per = H / G; return per < AS_T ? per : AS_T; }
+static int as_head_blocks(int H, int G) { const int per = H / G, hf = as_heads_per_tile(H, G); return (per + hf - 1) / hf; }
+
+extern "C" int64_t jl_attn_sweep_scratch_floats(int32_t n_tiles, int32_t H, int32_t G, int32_t Dv, int32_t splits) {
+    if (H <= 0 || G <= 0 || H % G) return 0;
+    return splits > 1 ? (int64_t)splits * n_tiles * G * as_head_blocks(H, G) * AS_T * (Dv + 2) : 0;
 }
 
-static bool as_fits(int dtype, int H, int G, int D, int Dv, int64_t k_ld) {
-    return dtype == JL_BF16 && G == 1 && H >= 1 && D % 8 == 0 && D <= 8 * AS_WAVES * AS_QSTEPS && Dv % 128 == 0 && Dv >= 128 && Dv <= 512 && Dv <= D &&
-           k_ld % 4 == 0;
+static bool as_fits(int dtype, int H, int G, int Gv, int D, int Dv, int64_t k_ld, int64_t v_ld, bool v_in_k) {
+    if (!(dtype == JL_BF16 && H >= 1 && G >= 1 && H % G == 0 && Gv >= 1 && G % Gv == 0 && D % 8 == 0 && D <= 8 * AS_WAVES * AS_QSTEPS && Dv % 32 == 0 &&
+          Dv >= 32 && Dv <= 512 && k_ld % 4 == 0 && v_ld % 4 == 0 && k_ld >= (int64_t)G * D))
+        return false;
+    if (v_in_k) return G == 1 && Dv <= D;
+    return v_ld >= (int64_t)Gv * Dv && as_lds_bytes(D, Dv, false) <= 150 * 1024;
 }
 
-extern "C" int jl_attn_shared_kv_tile_rows(int dtype, int32_t H, int32_t D, int32_t Dv, int64_t k_ld) {
-    if (!as_fits(dtype, H, 1, D, Dv, k_ld)) return 0;
-    const int hf = H < AS_T ? H : AS_T;
-    return AS_T / hf;
+extern "C" int jl_attn_sweep_tile_rows(int dtype, int32_t H, int32_t G, int32_t Gv, int32_t D, int32_t Dv, int64_t k_ld, int64_t v_ld, int32_t v_in_k) {
+    if (!as_fits(dtype, H, G, Gv > 0 ? Gv : G, D, Dv, k_ld, v_in_k ? k_ld : v_ld, v_in_k != 0)) return 0;
+    return AS_T / as_heads_per_tile(H, G);
 }
 
-extern "C" int jl_attn_shared_kv(const jl_attn_args *ap, void *stream) {
-    if (!ap) return jl_fail(JL_E_INVALID, "jl_attn_shared_kv: null arguments");
+extern "C" int jl_attn_sweep(const jl_attn_args *ap, void *stream) {
+    if (!ap) return jl_fail(JL_E_INVALID, "jl_attn_sweep: null arguments");
     jl_attn_args a = *ap;
     if (a.n_tiles <= 0) return JL_OK;
-    if (!a.q || !a.k_cache || !a.out || !a.block_tables || !a.tiles) return jl_fail(JL_E_INVALID, "jl_attn_shared_kv: null pointer");
-    if (a.k_ld <= 0) a.k_ld = a.D;
-    if (a.page_size <= 0 || a.k_ld < a.D || !as_fits(a.dtype, a.H, a.G, a.D, a.Dv, a.k_ld))
-        return jl_fail(JL_E_INVALID, "jl_attn_shared_kv: bfloat16, one key/value head, key width a multiple of 8 up to %d, value width 128 .. 512 in "
-                       "multiples of 128 and at most the key width", 8 * AS_WAVES * AS_QSTEPS);
-    if (a.v_cache && a.v_cache != a.k_cache) return jl_fail(JL_E_INVALID, "jl_attn_shared_kv: the values are the first Dv columns of the key rows");
-    const int hf = a.H < AS_T ? a.H : AS_T, tq = AS_T / hf;
-    if (a.TQ != tq) return jl_fail(JL_E_INVALID, "jl_attn_shared_kv: tiles of %d queries wanted (ask jl_attn_shared_kv_tile_rows)", tq);
-    const size_t lds = as_lds_bytes(a.D);
-    if (a.splits > 1 && (!a.scratch || a.splits > 64)) return jl_fail(JL_E_INVALID, "jl_attn_shared_kv: 2 .. 64 shares of the keys need a scratch");
-    const dim3 grid((unsigned)a.n_tiles, (unsigned)((a.H + hf - 1) / hf), (unsigned)(a.splits > 1 ? a.splits : 1));
+    if (!a.q || !a.k_cache || !a.v_cache || !a.out || !a.block_tables || !a.tiles) return jl_fail(JL_E_INVALID, "jl_attn_sweep: null pointer");
+    if (a.H <= 0 || a.G <= 0 || a.H % a.G || a.page_size <= 0) return jl_fail(JL_E_INVALID, "jl_attn_sweep: bad head counts or page size");
+    if (a.Gv <= 0) a.Gv = a.G;
+    if (a.k_ld <= 0) a.k_ld = (int64_t)a.G * a.D;
+    const bool v_in_k = a.v_cache == a.k_cache;
+    if (a.v_ld <= 0) a.v_ld = v_in_k ? a.k_ld : (int64_t)a.Gv * a.Dv;
+    if (!as_fits(a.dtype, a.H, a.G, a.Gv, a.D, a.Dv, a.k_ld, a.v_ld, v_in_k))
+        return jl_fail(JL_E_INVALID, "jl_attn_sweep: bfloat16, key width a multiple of 8 up to %d, value width a multiple of 32 up to 512, row strides in "
+                       "multiples of 4; values inside the key rows need one key head", 8 * AS_WAVES * AS_QSTEPS);
+    if (a.out_dtype != JL_OUT_SAME && a.out_dtype != JL_OUT_F32) return jl_fail(JL_E_INVALID, "jl_attn_sweep: unknown out_dtype");
+    const int hf = as_heads_per_tile(a.H, a.G), hb = as_head_blocks(a.H, a.G), tq = AS_T / hf;
+    if (a.TQ != tq) return jl_fail(JL_E_INVALID, "jl_attn_sweep: tiles of %d queries wanted (ask jl_attn_sweep_tile_rows)", tq);
+    if (a.splits > 1 && (!a.scratch || a.splits > 64)) return jl_fail(JL_E_INVALID, "jl_attn_sweep: 2 .. 64 shares of the keys need a scratch");
+    const size_t lds = as_lds_bytes(a.D, a.Dv, v_in_k);
+    const dim3 grid((unsigned)a.n_tiles, (unsigned)(a.G * hb), (unsigned)(a.splits > 1 ? a.splits : 1));
     hipStream_t st = (hipStream_t)stream;
 #define AS_CASE(NTV)                                                                                                              \
     case NTV: {                                                                                                                   \
-        auto kern = attn_shared_kv_kernel<NTV>;                                                                                   \
+        auto kern = attn_sweep_kernel<NTV>;                                                                                       \
         if (lds > 64 * 1024) {                                                                                                    \
             hipError_t e = hipFuncSetAttribute((const void *)kern, hipFuncAttributeMaxDynamicSharedMemorySize, (int)lds);         \
-            if (e != hipSuccess) return jl_fail(JL_E_LAUNCH, "jl_attn_shared_kv: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e)); \
+            if (e != hipSuccess) return jl_fail(JL_E_LAUNCH, "jl_attn_sweep: cannot get %zu bytes of LDS: %s", lds, hipGetErrorString(e)); \
         }                                                                                                                         \
-        kern<<<grid, AS_THREADS, lds, st>>>(a, hf, tq);                                                                           \
+        kern<<<grid, AS_THREADS, lds, st>>>(a, hf, tq, hb, v_in_k ? 1 : 0);                                                       \
         break;                                                                                                                    \
     }
-    switch (a.Dv / 128) {
+    switch ((a.Dv + 127) / 128) {
         AS_CASE(1) AS_CASE(2) AS_CASE(3) AS_CASE(4)
     }
 #undef AS_CASE
-    if (a.splits > 1) attn_shared_join_kernel<<<dim3(grid.x, grid.y), 256, 0, st>>>(a, hf, tq);
-    return jl_check_launch("attn_shared_kv_kernel");
+    if (a.splits > 1) attn_sweep_join_kernel<<<dim3(grid.x, grid.y), 256, 0, st>>>(a, hf, tq, hb);
+    return jl_check_launch("attn_sweep_kernel");
 }

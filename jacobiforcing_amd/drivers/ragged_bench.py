@@ -248,7 +248,8 @@ def kernel_table_vumalix(s, prompts, prompt_len, decode_batch, context, dtype=to
         # differential attention: norm + append, both maps' attention, combination
         proj = rnd(n, 2 * H * D + 2 * G * D + G * Dv)
         wq = rnd(D)
-        apart = 2 * H > LO.ATTN_MAX_HEADS_ONE_LAUNCH
+        sweep = LO.attn_sweep_tile_rows(dtype, 2 * H, 2 * G, D, Dv, kd, vd, G) > 0
+        apart = 2 * H > LO.ATTN_MAX_HEADS_ONE_LAUNCH and not sweep
         t_hn = timed(lambda: LO.head_norm_append(proj, (0, 2 * H * D, 2 * H * D + 2 * G * D), H, G, 2, D, Dv, wq, wq, 1e-6, 0.1, 256, batch, kd, vd, apart))
         row(f"{phase}.head_norm_append", t_hn, 2 * n * (2 * H * D + 2 * G * D + G * Dv) * es, 6.0 * n * (2 * H + 2 * G) * D, VECTOR_FLOPS)
         pk = rnd(n, KH * KD + 2 * KG * KD)
@@ -258,6 +259,8 @@ def kernel_table_vumalix(s, prompts, prompt_len, decode_batch, context, dtype=to
         q = LO.head_norm_append(proj, (0, 2 * H * D, 2 * H * D + 2 * G * D), H, G, 2, D, Dv, wq, wq, 1e-6, 0.1, 256, batch, kd, vd, apart)
 
         def diff_attn():
+            if sweep:
+                return LO.attn_sweep(q, kd, vd, batch, 2 * H, 2 * G, D, Dv, D ** -0.5, 0, value_heads=G, float_out=True)
             if not apart:
                 return LO.attn_window(q, None, kd, vd, batch, 2 * H, 2 * G, D, Dv, D ** -0.5, 0, 0, None, None, None, value_heads=G, float_out=True)
             return [LO.attn_window(q[mp], None, kd[:, mp * G * D:(mp + 1) * G * D], vd, batch, H, G, D, Dv, D ** -0.5, 0, 0, None, None, None, float_out=True)
@@ -279,8 +282,8 @@ def kernel_table_vumalix(s, prompts, prompt_len, decode_batch, context, dtype=to
         step = LO.ATTN_MAX_VALUE_WIDTH
 
         def latent_attn():
-            if LO.attn_shared_kv_tile_rows(dtype, LH, R + rd, R, lat.stride(0)):
-                return LO.attn_shared_kv(qf, lat, batch, LH, R + rd, R, 0.1, win)
+            if LO.attn_sweep_tile_rows(dtype, LH, 1, R + rd, R, lat, lat[:, :R]):
+                return LO.attn_sweep(qf, lat, lat[:, :R], batch, LH, 1, R + rd, R, 0.1, win)
             return [LO.attn_window(qf, None, lat, lat[:, c0:min(R, c0 + step)], batch, LH, 1, R + rd, min(R, c0 + step) - c0, 0.1, win, 0, None, None, None)
                     for c0 in range(0, R, step)]
         row(f"{phase}.attn_latent", timed(latent_attn), span_w * (R + rd) * es + n * LH * (2 * R + rd) * es, 2.0 * windowed * LH * (2 * R + rd), MATRIX_FLOPS)

@@ -18,6 +18,7 @@ from . import _native as N
 
 ATTN_SPLIT_BELOW_TILES, ATTN_SPLIT_WORKGROUPS = 128, 512     # attention: split a tile's keys while tiles x splits stays below ~2 per CU
 ATTN_MAX_HEADS_ONE_LAUNCH, ATTN_MAX_VALUE_WIDTH = 16, 128   # what the matrix-core attention kernel takes in one workgroup
+SWEEP_SPLIT_BELOW_GROUPS, SWEEP_SPLIT_WORKGROUPS = 512, 2048   # one-sweep attention: its workgroups are small (4 wavefronts, <= 32 rows)
 RETENTION_CHUNK = 64          # tokens per chunk when a long portion's recurrence is cut into chunks that run side by side
 
 
@@ -232,38 +233,46 @@ def attn_window(q: torch.Tensor, gate: Optional[torch.Tensor], k_cache: torch.Te
     return out
 
 
-def attn_shared_kv_tile_rows(dtype: torch.dtype, H: int, D: int, Dv: int, k_ld: int) -> int:
-    """Queries per tile of the shared key/value-head kernel for these sizes; 0 when it does not take them."""
-    if dtype != torch.bfloat16 or os.environ.get("JL_ATTN_NO_SHARED_KV"):                      # A/B switch for measurements
+def attn_sweep_tile_rows(dtype: torch.dtype, H: int, G: int, D: int, Dv: int, k_cache: torch.Tensor, v_cache: torch.Tensor, value_heads: int = 0) -> int:
+    """Queries per tile of the one-sweep kernel (heads in groups over a key head) for these sizes and pools; 0 when it does not
+    take them."""
+    if dtype != torch.bfloat16 or os.environ.get("JL_ATTN_NO_SWEEP"):                          # A/B switch for measurements
         return 0
-    return int(N.layers().jl_attn_shared_kv_tile_rows(_code(dtype), H, D, Dv, k_ld))
+    v_in_k = v_cache.data_ptr() == k_cache.data_ptr()
+    return int(N.layers().jl_attn_sweep_tile_rows(_code(dtype), H, G, value_heads or G, D, Dv, k_cache.stride(0), v_cache.stride(0), int(v_in_k)))
 
 
-def attn_shared_kv(q: torch.Tensor, pool: torch.Tensor, batch: RaggedBatch, H: int, D: int, Dv: int, scale: float, window: int) -> torch.Tensor:
-    """Attention of H query heads over one key/value head: q [N, H*D]; pool [tokens, >= D] whose rows hold the key (D columns)
-    with the value as its first Dv columns.  Returns [N, H*Dv].  Sizes as ``attn_shared_kv_tile_rows`` accepts them."""
+def attn_sweep(q: torch.Tensor, k_cache: torch.Tensor, v_cache: torch.Tensor, batch: RaggedBatch, H: int, G: int, D: int, Dv: int, scale: float,
+               window: int, value_heads: int = 0, float_out: bool = False) -> torch.Tensor:
+    """Attention without bias, head mixing or gate in one sweep on the matrix cores: q [N, H*D] bfloat16, pools as for
+    ``attn_window`` (column ranges of wider rows allowed); ``v_cache`` may be the first Dv columns of ``k_cache`` itself (one key
+    head whose rows hold the values: the latent pool).  Returns [N, H*Dv].  Sizes as ``attn_sweep_tile_rows`` accepts them."""
     _dev(q)
     n = q.shape[0]
-    _need(q.is_contiguous() and q.shape[1] == H * D and n == batch.N and pool.dtype == q.dtype and pool.dim() == 2 and pool.stride(1) == 1 and
-          pool.shape[1] >= D and Dv <= D, "attn_shared_kv: q [N, H*D] of the batch, pool rows of at least D columns")
-    _need(pool.shape[0] % batch.page_size == 0 and batch.max_page < pool.shape[0] // batch.page_size, "attn_shared_kv: a page lies outside the pool")
-    tq = attn_shared_kv_tile_rows(q.dtype, H, D, Dv, pool.stride(0))
-    _need(tq > 0, f"attn_shared_kv: heads={H} dim={D} vdim={Dv} are not sizes of this kernel")
+    Gv = value_heads or G
+    _need(q.is_contiguous() and q.shape[1] == H * D and n == batch.N and H % G == 0 and G % Gv == 0, "attn_sweep: q [N, H*D] of the batch")
+    _need(k_cache.dtype == q.dtype and v_cache.dtype == q.dtype and k_cache.dim() == 2 and v_cache.dim() == 2 and k_cache.shape[1] == G * D and
+          v_cache.shape[1] == Gv * Dv and k_cache.stride(1) == 1 and v_cache.stride(1) == 1 and k_cache.shape[0] == v_cache.shape[0],
+          "attn_sweep: pool dtype / widths")
+    _need(k_cache.shape[0] % batch.page_size == 0 and batch.max_page < k_cache.shape[0] // batch.page_size, "attn_sweep: a page lies outside the pool")
+    tq = attn_sweep_tile_rows(q.dtype, H, G, D, Dv, k_cache, v_cache, Gv)
+    _need(tq > 0, f"attn_sweep: heads={H} kv_heads={G} dim={D} vdim={Dv} are not sizes of this kernel")
     tiles = batch.tiles(tq)
-    out = torch.empty((n, H * Dv), dtype=q.dtype, device=q.device)
+    out = torch.empty((n, H * Dv), dtype=torch.float32 if float_out else q.dtype, device=q.device)
     # few tiles with many keys (decoding): share each tile's keys out over workgroups until the chip is full
-    groups = tiles.shape[0] * -(-H // 32)
+    groups = tiles.shape[0] * G * -(-(H // G) // 32)
     splits, scratch = 1, None
-    if groups < ATTN_SPLIT_BELOW_TILES:
+    if groups < SWEEP_SPLIT_BELOW_GROUPS:
         reach = batch.max_pos if window <= 0 else min(batch.max_pos, int(window) + tq)
-        splits = max(1, min(-(-reach // 64), ATTN_SPLIT_WORKGROUPS // groups, 64))
+        splits = max(1, min(-(-reach // 128), SWEEP_SPLIT_WORKGROUPS // groups, 64))
         if splits > 1:
-            scratch = torch.empty((int(N.layers().jl_attn_shared_kv_scratch_floats(tiles.shape[0], H, Dv, splits)),), dtype=torch.float32, device=q.device)
-    a = N.AttnArgs(q=q.data_ptr(), k_cache=pool.data_ptr(), v_cache=pool.data_ptr(), out=out.data_ptr(), block_tables=batch.tables.data_ptr(),
-                   tiles=tiles.data_ptr(), bt_stride=batch.tables.shape[1], n_tiles=tiles.shape[0], page_size=batch.page_size, H=H, G=1, D=D, Dv=Dv,
-                   window=int(window), TQ=tq, dtype=_code(q.dtype), scale=float(scale), n_rows=n, k_ld=pool.stride(0), Gv=1, splits=splits,
-                   scratch=scratch.data_ptr() if scratch is not None else None)
-    N.check_layers(N.layers().jl_attn_shared_kv(C.byref(a), _stream(q.device)), "jl_attn_shared_kv")
+            scratch = torch.empty((int(N.layers().jl_attn_sweep_scratch_floats(tiles.shape[0], H, G, Dv, splits)),), dtype=torch.float32, device=q.device)
+    a = N.AttnArgs(q=q.data_ptr(), k_cache=k_cache.data_ptr(), v_cache=v_cache.data_ptr(), out=out.data_ptr(), block_tables=batch.tables.data_ptr(),
+                   tiles=tiles.data_ptr(), bt_stride=batch.tables.shape[1], n_tiles=tiles.shape[0], page_size=batch.page_size, H=H, G=G, D=D, Dv=Dv,
+                   window=int(window), TQ=tq, dtype=_code(q.dtype), scale=float(scale), n_rows=n, k_ld=k_cache.stride(0), v_ld=v_cache.stride(0), Gv=Gv,
+                   splits=splits, scratch=scratch.data_ptr() if scratch is not None else None,
+                   out_dtype=N.JL_OUT_F32 if float_out else N.JL_OUT_SAME)
+    N.check_layers(N.layers().jl_attn_sweep(C.byref(a), _stream(q.device)), "jl_attn_sweep")
     return out
 
 

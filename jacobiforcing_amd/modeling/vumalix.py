@@ -224,11 +224,15 @@ class VumalixModel:
         H, G, D, Dv = int(m["heads"]), int(m["kv_heads"]), int(m["dim"]), int(m["vdim"])
         qt = m.get("q_temp") or {}
         proj = F.linear(h, w["w_in"])
-        apart = 2 * H > LO.ATTN_MAX_HEADS_ONE_LAUNCH
+        kp, vp, scale = cache.k[li], cache.v[li], float(m["scale"])
+        sweep = LO.attn_sweep_tile_rows(self.dtype, 2 * H, 2 * G, D, Dv, kp, vp, G) > 0
+        apart = 2 * H > LO.ATTN_MAX_HEADS_ONE_LAUNCH and not sweep
         q = LO.head_norm_append(proj, w["cols"], H, G, 2, D, Dv, w["q_norm"], w["k_norm"], eps, float(qt.get("coef", 0.0)), int(qt.get("every", 1)),
                                 batch, cache.k[li], cache.v[li], maps_apart=apart)
-        kp, vp, scale = cache.k[li], cache.v[li], float(m["scale"])
-        if not apart:   # one launch for both maps: 2H query heads over 2G key heads and G value heads, plain causal, float outputs
+        if sweep:       # bfloat16: both maps of all heads in one one-sweep launch (2G groups of H/G heads, G value heads)
+            a = LO.attn_sweep(q, kp, vp, batch, 2 * H, 2 * G, D, Dv, scale, 0, value_heads=G, float_out=True)
+            a1, a2 = a[:, :H * Dv], a[:, H * Dv:]
+        elif not apart:   # one launch for both maps: 2H query heads over 2G key heads and G value heads, plain causal, float outputs
             a = LO.attn_window(q, None, kp, vp, batch, 2 * H, 2 * G, D, Dv, scale, 0, 0, None, None, None, value_heads=G, float_out=True)
             a1, a2 = a[:, :H * Dv], a[:, H * Dv:]
         else:           # more heads than one workgroup takes: a launch per map over its own columns of the key rows
@@ -251,8 +255,8 @@ class VumalixModel:
         qf = LO.latent_q_pack(qa, q, H, D, R, rd, dims, batch, cos, sin)
         window, scale = int((m.get("mask") or {}).get("size", 0)), float(m["scale"])
         step = LO.ATTN_MAX_VALUE_WIDTH
-        if LO.attn_shared_kv_tile_rows(self.dtype, H, R + rd, R, pool.stride(0)):                   # bfloat16, latents of 128 .. 512: one sweep
-            o = LO.attn_shared_kv(qf, pool, batch, H, R + rd, R, scale, window)
+        if LO.attn_sweep_tile_rows(self.dtype, H, 1, R + rd, R, pool, pool[:, :R]):                 # bfloat16, latents in multiples of 32 up to 512
+            o = LO.attn_sweep(qf, pool, pool[:, :R], batch, H, 1, R + rd, R, scale, window)
             ov = torch.bmm(o.view(n, H, R).transpose(0, 1), w["w_uv"])
         elif R <= step or self.dtype != torch.bfloat16:
             o = LO.attn_window(qf, None, pool, pool[:, :R], batch, H, 1, R + rd, R, scale, window, 0, None, None, None)
