@@ -32,11 +32,78 @@ __global__ __launch_bounds__(256) void causal_conv_kernel(const float *__restric
     }
 }
 
+// The same for widths in multiples of four and up to eight taps: a workgroup walks CONV_ROWS consecutive rows, a thread owns four
+// channels and keeps the last TAPS - 1 inputs in registers, so that every input row is read once (plus the reach into the rows or
+// the tail before the workgroup's first row, and again where a new request starts).
+constexpr int CONV_ROWS = 8;
+template <typename T, int TAPS>
+__global__ __launch_bounds__(256) void causal_conv_rows_kernel(const float *__restrict__ x, const T *__restrict__ w, const int32_t *__restrict__ row_req,
+                                                                const int32_t *__restrict__ seq, float *tail, int64_t N, int W, T *__restrict__ out) {
+    constexpr int KEEP = TAPS - 1;
+    const int c = (blockIdx.y * 256 + threadIdx.x) * 4;
+    if (c >= W) return;
+    float wv[4][TAPS];
+#pragma unroll
+    for (int k = 0; k < 4; ++k)
+#pragma unroll
+        for (int j = 0; j < TAPS; ++j) wv[k][j] = ld_f(w + (int64_t)(c + k) * TAPS + j);
+    float4 win[KEEP > 0 ? KEEP : 1];
+    int prev_req = -1;
+    const int64_t n0 = (int64_t)blockIdx.x * CONV_ROWS;
+    for (int r = 0; r < CONV_ROWS && n0 + r < N; ++r) {
+        const int64_t n = n0 + r;
+        const int req = row_req[n];
+        const int32_t *rec = seq + 4 * (int64_t)req;
+        const int row0 = rec[0], count = rec[1], pos0 = rec[2], slot = rec[3];
+        const int t = (int)(n - row0);
+        if (req != prev_req) {                                  // the inputs before this row: earlier rows of the step, the tail, or nothing
+#pragma unroll
+            for (int s2 = 0; s2 < KEEP; ++s2) {
+                const int u = t - KEEP + s2;
+                float4 v = make_float4(0.f, 0.f, 0.f, 0.f);
+                if (u >= 0) v = *(const float4 *)(x + (int64_t)(row0 + u) * W + c);
+                else if (pos0 + u >= 0) v = *(const float4 *)(tail + ((int64_t)slot * KEEP + (KEEP + u)) * W + c);
+                win[s2] = v;
+            }
+            prev_req = req;
+        }
+        const float4 cur = *(const float4 *)(x + n * W + c);
+        float a0, a1, a2, a3;
+        a0 = cur.x + wv[0][KEEP] * cur.x; a1 = cur.y + wv[1][KEEP] * cur.y; a2 = cur.z + wv[2][KEEP] * cur.z; a3 = cur.w + wv[3][KEEP] * cur.w;
+#pragma unroll
+        for (int s2 = 0; s2 < KEEP; ++s2) {
+            a0 += wv[0][s2] * win[s2].x; a1 += wv[1][s2] * win[s2].y; a2 += wv[2][s2] * win[s2].z; a3 += wv[3][s2] * win[s2].w;
+        }
+        T *o = out + n * W + c;
+        st_f(o, a0); st_f(o + 1, a1); st_f(o + 2, a2); st_f(o + 3, a3);
+#pragma unroll
+        for (int s2 = 0; s2 + 1 < KEEP; ++s2) win[s2] = win[s2 + 1];
+        if (KEEP > 0) win[KEEP - 1] = cur;
+        if (count == 1 && KEEP > 0) {                           // a single row moves its request's tail on (its only reader is this thread)
+#pragma unroll
+            for (int s2 = 0; s2 < KEEP; ++s2) *(float4 *)(tail + ((int64_t)slot * KEEP + s2) * W + c) = win[s2];
+        }
+    }
+}
+
+template <typename T, int TAPS>
+static void conv_rows_launch(const float *x, const void *w, const int32_t *row_req, const int32_t *seq, float *tail, int64_t N, int W, void *out,
+                             hipStream_t st) {
+    const dim3 grid((unsigned)((N + CONV_ROWS - 1) / CONV_ROWS), (unsigned)((W / 4 + 255) / 256));
+    causal_conv_rows_kernel<T, TAPS><<<grid, 256, 0, st>>>(x, (const T *)w, row_req, seq, tail, N, W, (T *)out);
+}
+
 extern "C" int jl_causal_conv(const float *x, const void *w, int dtype, const int32_t *row_req, const int32_t *seq, float *tail,
                               int64_t N, int32_t W, int32_t taps, void *out, void *stream) {
     if (N <= 0) return JL_OK;
     if (!x || !w || !row_req || !seq || !out || W <= 0 || taps < 1 || taps > JL_CONV_MAX_TAPS || (taps > 1 && !tail))
         return jl_fail(JL_E_INVALID, "jl_causal_conv: null pointer, bad width or taps outside 1..%d", JL_CONV_MAX_TAPS);
+    if (W % 4 == 0 && taps <= 8) {
+#define CONV_CASE(TP) case TP: JL_DISPATCH(dtype, (conv_rows_launch<T, TP>(x, w, row_req, seq, tail, N, W, out, (hipStream_t)stream))); break
+        switch (taps) { CONV_CASE(1); CONV_CASE(2); CONV_CASE(3); CONV_CASE(4); CONV_CASE(5); CONV_CASE(6); CONV_CASE(7); CONV_CASE(8); }
+#undef CONV_CASE
+        return jl_check_launch("causal_conv_rows_kernel");
+    }
     JL_DISPATCH(dtype, causal_conv_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(x, (const T *)w, row_req, seq, tail, W, taps,
                                                                                                   (T *)out));
     return jl_check_launch("causal_conv_kernel");

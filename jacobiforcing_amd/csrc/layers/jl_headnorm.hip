@@ -39,6 +39,63 @@ __global__ __launch_bounds__(256) void head_norm_append_kernel(const T *__restri
         for (int c = threadIdx.x; c < GDv; c += 256) v_cache[sl * GDv + c] = row[v_col + c];
 }
 
+// four elements at a time (8 bytes of bfloat16, 16 of float)
+__device__ __forceinline__ void ld4(const float *p, float (&v)[4]) { const float4 t = *(const float4 *)p; v[0] = t.x; v[1] = t.y; v[2] = t.z; v[3] = t.w; }
+__device__ __forceinline__ void ld4(const bf16_t *p, float (&v)[4]) {
+    const uint2 t = *(const uint2 *)p;
+    v[0] = __uint_as_float(t.x << 16); v[1] = __uint_as_float(t.x & 0xffff0000u); v[2] = __uint_as_float(t.y << 16); v[3] = __uint_as_float(t.y & 0xffff0000u);
+}
+__device__ __forceinline__ void st4(float *p, const float (&v)[4]) { *(float4 *)p = make_float4(v[0], v[1], v[2], v[3]); }
+__device__ __forceinline__ void st4(bf16_t *p, const float (&v)[4]) {
+    bf16_t h[4];
+#pragma unroll
+    for (int i = 0; i < 4; ++i) st_f(h + i, v[i]);
+    *(uint2 *)p = make_uint2((uint32_t)h[0] | ((uint32_t)h[1] << 16), (uint32_t)h[2] | ((uint32_t)h[3] << 16));
+}
+
+// The same with LPV lanes per D-vector (a power of two, 4 * LPV >= D, D % 4 == 0, every column offset and row stride a multiple of
+// four): a wavefront normalises 64 / LPV vectors at a time, four elements per lane and load.
+template <typename T>
+__global__ __launch_bounds__(256) void head_norm_append_vec_kernel(const T *__restrict__ proj, int64_t ld, int q_col, int k_col, int v_col, int H, int G,
+                                                                    int M, int D, int GDv, const T *__restrict__ wq, const T *__restrict__ wk, float eps,
+                                                                    float t_coef, int t_every, const int32_t *__restrict__ pos, T *__restrict__ q_out,
+                                                                    int64_t q_map_stride, T *__restrict__ k_cache, T *__restrict__ v_cache,
+                                                                    const int64_t *__restrict__ slot, int LPV) {
+    const int64_t n = blockIdx.x;
+    const T *row = proj + n * ld;
+    const int sub = threadIdx.x & (LPV - 1), group = threadIdx.x / LPV, groups = 256 / LPV;
+    const int64_t sl = slot[n];
+    float temp = 1.0f;
+    if (t_coef != 0.f) temp = 1.0f + t_coef * logf((float)((pos[n] + 1) / t_every + 1));
+    const int nq = H * M, nk = G * M, d = 4 * sub;
+    for (int v0 = 0; v0 < nq + nk; v0 += groups) {              // every lane takes part in the shuffles of its round
+        const int vec = v0 + group;
+        const bool live = vec < nq + nk && d < D;
+        const bool is_q = vec < nq;
+        const int idx = is_q ? vec : vec - nq;
+        const int head = idx / M, map = idx - head * M;
+        float x[4] = {0.f, 0.f, 0.f, 0.f};
+        if (live) ld4(row + (is_q ? q_col : k_col) + (int64_t)idx * D + d, x);
+        float ss = x[0] * x[0] + x[1] * x[1] + x[2] * x[2] + x[3] * x[3];
+        for (int off = LPV >> 1; off > 0; off >>= 1) ss += __shfl_xor(ss, off, 64);
+        if (!live) continue;
+        const float r = 1.0f / sqrtf(ss / (float)D + eps) * (is_q ? temp : 1.0f);
+        float g[4];
+        ld4((is_q ? wq : wk) + d, g);
+#pragma unroll
+        for (int i = 0; i < 4; ++i) x[i] = x[i] * r * g[i];
+        if (is_q) {
+            T *dst = q_map_stride ? q_out + map * q_map_stride + n * ((int64_t)H * D) + (int64_t)head * D
+                                  : q_out + n * ((int64_t)nq * D) + ((int64_t)map * H + head) * D;
+            st4(dst + d, x);
+        } else if (sl >= 0) {
+            st4(k_cache + sl * ((int64_t)nk * D) + ((int64_t)map * G + head) * D + d, x);
+        }
+    }
+    if (sl >= 0)
+        for (int c = threadIdx.x; c < GDv; c += 256) v_cache[sl * GDv + c] = row[v_col + c];
+}
+
 extern "C" int jl_head_norm_append(const void *proj, int dtype, int64_t N, int64_t ld, int32_t q_col, int32_t k_col, int32_t v_col, int32_t H,
                                    int32_t G, int32_t M, int32_t D, int32_t Dv, const void *wq, const void *wk, float eps, float t_coef,
                                    int32_t t_every, const int32_t *pos, void *q_out, int32_t maps_apart, void *k_cache, void *v_cache,
@@ -48,6 +105,14 @@ extern "C" int jl_head_norm_append(const void *proj, int dtype, int64_t N, int64
     if (H <= 0 || G <= 0 || M <= 0 || D <= 0 || Dv <= 0 || q_col + (int64_t)H * M * D > ld || k_col + (int64_t)G * M * D > ld || v_col + (int64_t)G * Dv > ld)
         return jl_fail(JL_E_INVALID, "jl_head_norm_append: columns do not fit the row stride");
     if (t_coef != 0.f && (!pos || t_every <= 0)) return jl_fail(JL_E_INVALID, "jl_head_norm_append: a query temperature needs positions and a period >= 1");
+    if (D % 4 == 0 && D <= 256 && ld % 4 == 0 && q_col % 4 == 0 && k_col % 4 == 0) {
+        int lpv = 1;
+        while (4 * lpv < D) lpv <<= 1;
+        JL_DISPATCH(dtype, head_norm_append_vec_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(
+                               (const T *)proj, ld, q_col, k_col, v_col, H, G, M, D, G * Dv, (const T *)wq, (const T *)wk, eps, t_coef, t_every, pos,
+                               (T *)q_out, maps_apart ? N * (int64_t)H * D : 0, (T *)k_cache, (T *)v_cache, slot, lpv));
+        return jl_check_launch("head_norm_append_vec_kernel");
+    }
     JL_DISPATCH(dtype, head_norm_append_kernel<T><<<dim3((unsigned)N), 256, 0, (hipStream_t)stream>>>(
                            (const T *)proj, ld, q_col, k_col, v_col, H, G, M, D, G * Dv, (const T *)wq, (const T *)wk, eps, t_coef, t_every, pos,
                            (T *)q_out, maps_apart ? N * (int64_t)H * D : 0, (T *)k_cache, (T *)v_cache, slot));

@@ -47,8 +47,12 @@ class VumalixConfig:
         return len(self.layers)
 
     def weights_layer(self, i: int) -> int:
-        """The layer whose tensors layer i uses (itself unless it borrows)."""
-        return int(self.layers[i].get("weights_of", i))
+        """The layer whose tensors layer i uses (itself unless it borrows; a borrowed layer that borrows in turn is followed)."""
+        seen = set()
+        while self.layers[i].get("weights_of") is not None and i not in seen:
+            seen.add(i)
+            i = int(self.layers[i]["weights_of"])
+        return i
 
     @classmethod
     def from_dict(cls, d: Dict[str, Any]) -> "VumalixConfig":
@@ -63,9 +67,11 @@ class VumalixConfig:
                 raise ValueError(f"layer {i}: unknown feed-forward {L['mlp'].get('kind')!r}")
             j = L.get("weights_of")
             if j is not None:
-                j = int(j)
-                if not 0 <= j < len(layers) or "weights_of" in layers[j] or layers[j]["type"] != L["type"]:
-                    raise ValueError(f"layer {i}: weights_of {j} must name a layer of the same type that owns its tensors")
+                j, hops = int(j), 0
+                while 0 <= j < len(layers) and layers[j].get("weights_of") is not None and hops < len(layers):
+                    j, hops = int(layers[j]["weights_of"]), hops + 1
+                if not 0 <= j < len(layers) or layers[j].get("weights_of") is not None or layers[j]["type"] != L["type"]:
+                    raise ValueError(f"layer {i}: weights_of must lead to a layer of the same type that owns its tensors")
             m = L["mixer"]
             if L["type"] == "attention" and int(m["heads"]) % int(m["kv_heads"]):
                 raise ValueError(f"layer {i}: {m['heads']} heads over {m['kv_heads']} key/value heads")
@@ -225,18 +231,19 @@ class VumalixModel:
         qt = m.get("q_temp") or {}
         proj = F.linear(h, w["w_in"])
         kp, vp, scale = cache.k[li], cache.v[li], float(m["scale"])
+        window = int((m.get("mask") or {}).get("size", 0))                                          # none in the design: plain causal
         sweep = LO.attn_sweep_tile_rows(self.dtype, 2 * H, 2 * G, D, Dv, kp, vp, G) > 0
         apart = 2 * H > LO.ATTN_MAX_HEADS_ONE_LAUNCH and not sweep
         q = LO.head_norm_append(proj, w["cols"], H, G, 2, D, Dv, w["q_norm"], w["k_norm"], eps, float(qt.get("coef", 0.0)), int(qt.get("every", 1)),
                                 batch, cache.k[li], cache.v[li], maps_apart=apart)
         if sweep:       # bfloat16: both maps of all heads in one one-sweep launch (2G groups of H/G heads, G value heads)
-            a = LO.attn_sweep(q, kp, vp, batch, 2 * H, 2 * G, D, Dv, scale, 0, value_heads=G, float_out=True)
+            a = LO.attn_sweep(q, kp, vp, batch, 2 * H, 2 * G, D, Dv, scale, window, value_heads=G, float_out=True)
             a1, a2 = a[:, :H * Dv], a[:, H * Dv:]
         elif not apart:   # one launch for both maps: 2H query heads over 2G key heads and G value heads, plain causal, float outputs
-            a = LO.attn_window(q, None, kp, vp, batch, 2 * H, 2 * G, D, Dv, scale, 0, 0, None, None, None, value_heads=G, float_out=True)
+            a = LO.attn_window(q, None, kp, vp, batch, 2 * H, 2 * G, D, Dv, scale, window, 0, None, None, None, value_heads=G, float_out=True)
             a1, a2 = a[:, :H * Dv], a[:, H * Dv:]
         else:           # more heads than one workgroup takes: a launch per map over its own columns of the key rows
-            a1, a2 = (LO.attn_window(q[mp], None, kp[:, mp * G * D:(mp + 1) * G * D], vp, batch, H, G, D, Dv, scale, 0, 0, None, None, None,
+            a1, a2 = (LO.attn_window(q[mp], None, kp[:, mp * G * D:(mp + 1) * G * D], vp, batch, H, G, D, Dv, scale, window, 0, None, None, None,
                                      float_out=True) for mp in range(2))
         return LO.diff_combine(a1, a2, H, Dv, w["lam"], eps, 1.0 - float(m["diff"]), self.dtype)
 

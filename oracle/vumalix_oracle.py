@@ -55,15 +55,17 @@ def differential_attention(h, P, m, eps):
     k = unit_rms((h @ P["mix.k"].T).view(T, G, 2, D), eps) * P["mix.k.norm"]
     v = (h @ P["mix.v"].T).view(T, G, Dv)
     lam = differential_lambda(P, m["diff"])
+    size = (m.get("mask") or {}).get("size", 0) or T + 1           # the design's layers have no window; one that has is honoured
     out = torch.zeros(T, H, Dv, dtype=h.dtype)
     for i in range(T):
         temp = query_temperature(i, qt["coef"], qt["every"])
+        lo = max(0, i - size + 1)
         for hh in range(H):
             c = hh // (H // G)
             maps = []
             for mp in range(2):
-                s = (k[:i + 1, c, mp] @ (q[i, hh, mp] * temp)) * m["scale"]
-                maps.append(torch.softmax(s, 0) @ v[:i + 1, c])
+                s = (k[lo:i + 1, c, mp] @ (q[i, hh, mp] * temp)) * m["scale"]
+                maps.append(torch.softmax(s, 0) @ v[lo:i + 1, c])
             o = maps[0] - lam * maps[1]
             out[i, hh] = unit_rms(o, eps) * (1.0 - m["diff"])
     return out.reshape(T, H * Dv) @ P["mix.o"].T

@@ -103,6 +103,9 @@ def test_config_rejects_what_the_design_does_not_have():
     bad["layers"][1]["mlp"]["kind"] = "moe"
     with pytest.raises(ValueError):
         VX.VumalixConfig.from_dict(bad)
+    chain = shape_a()
+    chain["layers"][4]["weights_of"] = 2                                                       # borrows from a layer that borrows: followed
+    assert VX.VumalixConfig.from_dict(dict(chain, layers=chain["layers"][:3] + [chain["layers"][0] | {"weights_of": 2}])).weights_layer(3) == 0
     bad = shape_a()
     bad["canon"]["taps"] = 0
     with pytest.raises(ValueError):
@@ -257,29 +260,33 @@ def test_output_norm_residual_and_activation(W):
 
 
 @gpu
-@pytest.mark.parametrize("taps,cuts", [(4, [9]), (4, [1, 1, 1, 2, 4]), (3, [2, 7]), (7, [3, 2, 1, 3]), (1, [4, 5]), (2, [1] * 9)])
+@pytest.mark.parametrize("taps,cuts", [(4, [9]), (4, [1, 1, 1, 2, 4]), (3, [2, 7]), (7, [3, 2, 1, 3]), (1, [4, 5]), (2, [1] * 9), (9, [3, 5, 1, 1, 12]),
+                                       (5, [1, 19, 2, 1, 1])])
 def test_convolution_carries_its_tail_across_steps(taps, cuts):
-    """A request cut into portions shorter and longer than the taps, beside a second request that starts later in a used slot."""
+    """A request cut into portions shorter and longer than the taps, beside a second request that starts later in a used slot.
+    Width 70 takes the kernel with a channel per thread, 72 the one with four channels per thread and the inputs kept in registers
+    (up to eight taps)."""
     from jacobiforcing_amd import layer_ops as LO
-    W, T = 70, sum(cuts)
-    g = torch.Generator().manual_seed(taps)
-    xa, xb, w = torch.randn(T, W, generator=g), torch.randn(T, W, generator=g), torch.randn(W, taps, generator=g)
-    want_a, want_b = O.time_conv_mix(xa.double(), w.double()), O.time_conv_mix(xb[:T - cuts[0]].double(), w.double())
-    tail = torch.full((3, taps - 1, W), 1e4).cuda() if taps > 1 else None
-    got_a, got_b, done = [], [], 0
-    for s, c in enumerate(cuts):
-        counts, starts, slots, rows = [c], [done], [2], [xa[done:done + c]]
-        if s > 0:                                                                              # the second request is one portion behind
-            counts.append(c); starts.append(done - cuts[0]); slots.append(0); rows.append(xb[done - cuts[0]:done - cuts[0] + c])
-        b = LO.RaggedBatch.build(counts, starts, slots, [[0, 1, 2, 3]] * len(counts), 16, "cuda")
-        out = LO.causal_conv(torch.cat(rows).cuda(), w.cuda(), b, tail).cpu()
-        got_a.append(out[:c])
-        if s > 0:
-            got_b.append(out[c:])
-        done += c
-    assert rel_err(torch.cat(got_a), want_a) < 1e-6
-    if got_b:
-        assert rel_err(torch.cat(got_b), want_b[:sum(cuts[1:])]) < 1e-6
+    for W in (70, 72):
+        T = sum(cuts)
+        g = torch.Generator().manual_seed(taps)
+        xa, xb, w = torch.randn(T, W, generator=g), torch.randn(T, W, generator=g), torch.randn(W, taps, generator=g)
+        want_a, want_b = O.time_conv_mix(xa.double(), w.double()), O.time_conv_mix(xb[:T - cuts[0]].double(), w.double())
+        tail = torch.full((3, taps - 1, W), 1e4).cuda() if taps > 1 else None
+        got_a, got_b, done = [], [], 0
+        for s, c in enumerate(cuts):
+            counts, starts, slots, rows = [c], [done], [2], [xa[done:done + c]]
+            if s > 0:                                                                          # the second request is one portion behind
+                counts.append(c); starts.append(done - cuts[0]); slots.append(0); rows.append(xb[done - cuts[0]:done - cuts[0] + c])
+            b = LO.RaggedBatch.build(counts, starts, slots, [[0, 1, 2, 3]] * len(counts), 16, "cuda")
+            out = LO.causal_conv(torch.cat(rows).cuda(), w.cuda(), b, tail).cpu()
+            got_a.append(out[:c])
+            if s > 0:
+                got_b.append(out[c:])
+            done += c
+        assert rel_err(torch.cat(got_a), want_a) < 1e-6, W
+        if got_b:
+            assert rel_err(torch.cat(got_b), want_b[:sum(cuts[1:])]) < 1e-6, W
 
 
 @gpu
@@ -537,6 +544,58 @@ def test_long_decoding_keeps_the_tails_and_the_window():
     rb = Rig(shape_b(), seed=29, pages=64, dtype=torch.bfloat16)
     gb = torch.cat([rb.step([("r", t[:20])])] + [rb.step([("r", [x])]) for x in t[20:]])
     assert rel_err(gb, want) < BF16_TOL
+
+
+def random_shape(seed):
+    """A random configuration: layer order, head counts, sizes (multiples of eight and not), windows from one token to longer than
+    the sequence, taps, constants; some layers borrow an earlier layer's weights."""
+    r = random.Random(seed)
+    layers = []
+    for i in range(r.choice([2, 3, 4])):
+        mlp = None if r.random() < 0.25 else dense(r.choice([8, 24, 40, 100]))
+        same = [j for j, L in enumerate(layers) if "weights_of" not in L]
+        if same and r.random() < 0.3:
+            j = r.choice(same)
+            layers.append(dict(json.loads(json.dumps(layers[j])), weights_of=j))
+            continue
+        if r.random() < 0.5:
+            kv = r.choice([1, 2, 3, 4])
+            layers.append(dict(diff_attn(heads=kv * r.choice([1, 2, 3, 5]), kv=kv, dim=r.choice([8, 16, 20, 24, 32, 64]), vdim=r.choice([8, 16, 32, 40, 64, 96]),
+                                         diff=r.choice([0.1, 0.25, 0.5, 0.9]), coef=r.choice([0.0, 0.3, 1.0]), every=r.choice([1, 3, 16, 64]),
+                                         scale=r.choice([0.1, 0.25, 0.5])), mlp=mlp))
+            if r.random() < 0.2:
+                layers[-1]["mixer"]["mask"] = {"size": r.choice([3, 12])}
+        else:
+            rd = r.choice([4, 8, 16])
+            layers.append(dict(latent(heads=r.choice([1, 2, 5, 8, 16, 33]), dim=r.choice([8, 16, 24]), rot_dim=rd, vdim=r.choice([8, 16, 24]),
+                                      kv_rank=r.choice([16, 32, 40, 64, 96, 128]), q_rank=r.choice([8, 24]), size=r.choice([1, 2, 5, 8, 9, 17, 40, 1000]),
+                                      base=r.choice([100.0, 10000.0]), scale=r.choice([0.1, 0.25])), mlp=mlp))
+    return make_cfg(layers, width=r.choice([32, 48, 64, 72, 100]), vocab=r.choice([17, 64, 131]), taps=r.choice([1, 2, 3, 4, 6]), eps=r.choice([1e-5, 1e-6]))
+
+
+@gpu
+@pytest.mark.parametrize("seed", range(12))
+def test_random_configurations_in_a_mixed_schedule(seed):
+    """Two requests cut at random into portions and single tokens, side by side from poisoned pools and tails, float32 and bfloat16."""
+    cfg = random_shape(seed)
+    r = random.Random(100 + seed)
+    V = cfg["vocab"]
+    a, b = toks(45, V, seed), toks(29, V, seed + 50)
+    for dtype, tol in ((torch.float32, F32_TOL), (torch.bfloat16, 2 * BF16_TOL)):
+        rig = Rig(cfg, seed=seed, dtype=dtype, pages=32)
+        want_a, want_b = rig.oracle(a)[0], rig.oracle(b)[0]
+        rig.poison()
+        got_a, got_b, ia, ib = [], [], 0, 0
+        while ia < len(a) or ib < len(b):
+            na = min(len(a) - ia, r.choice([1, 1, 2, 3, 7, 16]))
+            nb = min(len(b) - ib, r.choice([0, 1, 1, 2, 5, 11])) if ia > 6 else 0
+            entries = ([("a", a[ia:ia + na])] if na else []) + ([("b", b[ib:ib + nb])] if nb else [])
+            if not entries:
+                entries, nb = [("b", b[ib:ib + 1])], 1
+            out = rig.step(entries)
+            got_a.append(out[:na]); got_b.append(out[na:])
+            ia += na; ib += nb
+        assert rel_err(torch.cat(got_a), want_a) < tol and rel_err(torch.cat(got_b), want_b) < tol, (seed, dtype, cfg)
 
 
 def _write_model(tmp_path, cfg_dict, tensors):
