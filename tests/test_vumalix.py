@@ -356,7 +356,7 @@ def test_portions_of_any_size(cuts):
 
 @gpu
 @pytest.mark.parametrize("H,G,D,Dv", [(4, 2, 32, 48), (8, 8, 64, 32), (3, 1, 24, 40), (2, 1, 128, 128), (12, 4, 16, 16), (16, 4, 64, 128), (5, 5, 40, 96),
-                                      (40, 1, 16, 32), (6, 2, 24, 160)])
+                                      (40, 1, 16, 32), (6, 2, 24, 160), (2, 1, 256, 512)])
 def test_bfloat16_differential_attention_alone(H, G, D, Dv):
     """The bfloat16 paths — the one-sweep kernel where the value width is a multiple of 32 (groups of 1, 3, 4 and 40 heads), the
     two-sweep matrix-core kernel, one launch per map with many heads, the plain kernel for the rest — on a prompt of several tiles,
